@@ -1,0 +1,75 @@
+// Shared device/host helpers for the gfx950 kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "../../include/gptoss_mi355.h"
+
+namespace gptoss {
+
+// ---- error plumbing (host) -------------------------------------------------------------------
+void set_error(const char *fmt, ...);
+int fail(int code, const char *fmt, ...);
+
+#define GPTOSS_REQUIRE(cond, code, ...)                 \
+  do {                                                  \
+    if (!(cond)) return ::gptoss::fail(code, __VA_ARGS__); \
+  } while (0)
+
+#define GPTOSS_HIP(call)                                                                       \
+  do {                                                                                         \
+    hipError_t err__ = (call);                                                                 \
+    if (err__ != hipSuccess)                                                                   \
+      return ::gptoss::fail(GPTOSS_ERR_HIP, "%s: %s (%s:%d)", #call, hipGetErrorString(err__), \
+                            __FILE__, __LINE__);                                               \
+  } while (0)
+
+#define GPTOSS_LAUNCH_CHECK(name)                                                           \
+  do {                                                                                      \
+    hipError_t err__ = hipGetLastError();                                                   \
+    if (err__ != hipSuccess)                                                                \
+      return ::gptoss::fail(GPTOSS_ERR_HIP, "launch %s: %s", name, hipGetErrorString(err__)); \
+  } while (0)
+
+static inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
+static inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+static inline int cdiv(int a, int b) { return (a + b - 1) / b; }
+
+// ---- device types ----------------------------------------------------------------------------
+typedef uint16_t bf16_t;  // raw bf16 bits
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int WAVE = 64;
+
+__device__ __forceinline__ float bf16_to_f32(bf16_t b) { return __uint_as_float(((uint32_t)b) << 16); }
+
+// round-to-nearest-even; NaN stays NaN
+__device__ __forceinline__ bf16_t f32_to_bf16(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x40);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (bf16_t)(u >> 16);
+}
+
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  return (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
+}
+
+__device__ __forceinline__ bf16x8 as_bf16x8(u32x4 v) {
+  union {
+    u32x4 u;
+    bf16x8 b;
+  } c;
+  c.u = v;
+  return c.b;
+}
+
+__device__ __forceinline__ int lane_id() { return threadIdx.x & (WAVE - 1); }
+
+}  // namespace gptoss

@@ -1,0 +1,30 @@
+// Internal interface of the grouped/dense GEMM kernels (moe_gemm.hip).
+#pragma once
+#include "common.hpp"
+
+namespace gptoss {
+
+enum { EPI_F32 = 0, EPI_SWIGLU = 1, EPI_BF16 = 2 };
+
+struct GemmParams {
+  const bf16_t *A;     // activations, row-major [*, K]
+  const int *row_ids;  // gather: sorted pair ids (row of A = id / top_k); else unused
+  int top_k;
+  const bf16_t *W;     // packed weights, per-matrix stride N*K
+  const float *bias;   // [n_mat, N] or nullptr
+  void *out;           // EPI_F32: float [*, N]; EPI_SWIGLU: bf16 [*, N/2]; EPI_BF16: bf16 [*, N]
+  const int *tiles;    // {n_tiles, (mat,row0,rows)*} or nullptr for a dense problem
+  int dense_rows;      // rows of the dense problem when tiles == nullptr
+  int N, K;
+  int n_col_tiles;     // cdiv(N, 256)
+  float limit;         // SwiGLU clamp
+};
+
+// rows_per_tile in {32,64,128,256}; max_tiles bounds the number of (mat,row-tile) items.
+int run_gemm(const GemmParams &p, bool gather, int epi, int rows_per_tile, int max_tiles,
+             hipStream_t s);
+int run_combine(const float *y2, const float *topk_w, const int *inv_perm, float *out, int B, int H,
+                int k, int accumulate, hipStream_t s);
+int moe_rows_per_tile(int B, int k, int E);
+
+}  // namespace gptoss

@@ -1,0 +1,141 @@
+// Host side of the MoE block: workspace layout and the launch sequence
+// router GEMM -> top-k/softmax -> stable grouping + tile list -> grouped GEMM1 (+gather, +SwiGLU)
+// -> grouped GEMM2 -> ordered weighted combine.  Nothing here synchronises or allocates.
+#include "common.hpp"
+#include "gemm.hpp"
+
+namespace gptoss {
+
+struct MoeWorkspace {
+  float *logits, *topk_w;
+  int *topk_i, *expert_offsets, *sorted_pair_ids, *inv_perm, *tiles;
+  bf16_t *act;
+  float *y2;
+  size_t bytes;
+};
+
+static MoeWorkspace carve(void *base, int B, int E, int k, int H, int I) {
+  MoeWorkspace w;
+  size_t off = 0;
+  auto take = [&](size_t n) {
+    size_t o = off;
+    off += align_up(n, 256);
+    return reinterpret_cast<unsigned char *>(base) + o;
+  };
+  const size_t P = (size_t)B * k;
+  w.logits = (float *)take((size_t)B * E * 4);
+  w.topk_w = (float *)take(P * 4);
+  w.topk_i = (int *)take(P * 4);
+  w.expert_offsets = (int *)take((size_t)(E + 1) * 4);
+  w.sorted_pair_ids = (int *)take(P * 4);
+  w.inv_perm = (int *)take(P * 4);
+  w.tiles = (int *)take((1 + 3 * (P / 32 + E)) * 4);
+  w.act = (bf16_t *)take(P * I * 2);
+  w.y2 = (float *)take(P * H * 4);
+  w.bytes = off;
+  return w;
+}
+
+int moe_rows_per_tile(int B, int k, int E) {
+  long long avg = ((long long)B * k + E - 1) / E;
+  if (avg <= 21) return 32;
+  if (avg <= 42) return 64;
+  if (avg <= 85) return 128;
+  return 256;
+}
+
+static int check_moe(const gptoss_moe_weights *w, const void *t, int B, float *out, void *ws,
+                     size_t ws_bytes) {
+  GPTOSS_REQUIRE(w && t && out, GPTOSS_ERR_NULL, "moe_forward: null pointer");
+  GPTOSS_REQUIRE(w->w_router && w->w1 && w->w2, GPTOSS_ERR_NULL, "moe_forward: null weight pointer");
+  const int E = w->n_experts, k = w->top_k, H = w->hidden, I = w->intermediate;
+  GPTOSS_REQUIRE(B >= 0 && E >= 1 && E <= 256 && k >= 1 && k <= 8 && k <= E, GPTOSS_ERR_DIM,
+                 "moe_forward: need 1 <= k <= min(8,E), E <= 256 (B=%d E=%d k=%d)", B, E, k);
+  GPTOSS_REQUIRE(H > 0 && I > 0 && H % 64 == 0 && I % 64 == 0, GPTOSS_ERR_DIM,
+                 "moe_forward: need hidden %% 64 == 0 and intermediate %% 64 == 0 (H=%d I=%d)", H, I);
+  GPTOSS_REQUIRE((long long)B * k * (long long)(H > I ? H : I) < (1ll << 31), GPTOSS_ERR_DIM,
+                 "moe_forward: B*k*max(H,I) must stay below 2^31");
+  GPTOSS_REQUIRE(aligned(t, 16) && aligned(out, 16) && aligned(w->w1, 16) && aligned(w->w2, 16) &&
+                     aligned(w->w_router, 16),
+                 GPTOSS_ERR_ALIGN, "moe_forward: pointers must be 16-byte aligned");
+  GPTOSS_REQUIRE(ws != nullptr && aligned(ws, 256), GPTOSS_ERR_WORKSPACE,
+                 "moe_forward: workspace missing or not 256-byte aligned");
+  size_t need = gptoss_moe_workspace_bytes(B, E, k, H, I);
+  GPTOSS_REQUIRE(ws_bytes >= need, GPTOSS_ERR_WORKSPACE,
+                 "moe_forward: workspace has %zu bytes, needs %zu", ws_bytes, need);
+  return GPTOSS_OK;
+}
+
+}  // namespace gptoss
+
+using namespace gptoss;
+
+extern "C" size_t gptoss_moe_workspace_bytes(int B, int E, int k, int H, int I) {
+  if (B < 0 || E <= 0 || k <= 0 || H <= 0 || I <= 0) return 0;
+  return carve(nullptr, B, E, k, H, I).bytes;
+}
+
+extern "C" int gptoss_moe_workspace_views(void *workspace, int B, int E, int k, int H, int I,
+                                          float **logits, float **topk_w, int **topk_i,
+                                          int **expert_offsets, int **sorted_pair_ids,
+                                          int **inv_perm) {
+  GPTOSS_REQUIRE(workspace, GPTOSS_ERR_NULL, "moe_workspace_views: null workspace");
+  GPTOSS_REQUIRE(B >= 0 && E > 0 && k > 0 && H > 0 && I > 0, GPTOSS_ERR_DIM,
+                 "moe_workspace_views: bad dimensions");
+  MoeWorkspace w = carve(workspace, B, E, k, H, I);
+  if (logits) *logits = w.logits;
+  if (topk_w) *topk_w = w.topk_w;
+  if (topk_i) *topk_i = w.topk_i;
+  if (expert_offsets) *expert_offsets = w.expert_offsets;
+  if (sorted_pair_ids) *sorted_pair_ids = w.sorted_pair_ids;
+  if (inv_perm) *inv_perm = w.inv_perm;
+  return GPTOSS_OK;
+}
+
+extern "C" int gptoss_moe_forward(const gptoss_moe_weights *w, const void *t, int B, float *out,
+                                  int accumulate, void *workspace, size_t workspace_bytes,
+                                  void *stream) {
+  int rc = check_moe(w, t, B, out, workspace, workspace_bytes);
+  if (rc != GPTOSS_OK) return rc;
+  if (B == 0) return GPTOSS_OK;
+  const int E = w->n_experts, k = w->top_k, H = w->hidden, I = w->intermediate;
+  hipStream_t s = (hipStream_t)stream;
+  MoeWorkspace ws = carve(workspace, B, E, k, H, I);
+  const int rpt = moe_rows_per_tile(B, k, E);
+  const int max_tiles = gptoss_moe_max_tiles(B, k, E, rpt);
+
+  rc = gptoss_router_gemm(t, w->w_router, w->b_router, ws.logits, B, H, E, stream);
+  if (rc != GPTOSS_OK) return rc;
+  rc = gptoss_moe_route(ws.logits, B, E, k, ws.topk_w, ws.topk_i, ws.expert_offsets,
+                        ws.sorted_pair_ids, ws.inv_perm, ws.tiles, rpt, stream);
+  if (rc != GPTOSS_OK) return rc;
+
+  GemmParams g1{};
+  g1.A = (const bf16_t *)t;
+  g1.row_ids = ws.sorted_pair_ids;
+  g1.top_k = k;
+  g1.W = (const bf16_t *)w->w1;
+  g1.bias = w->b1;
+  g1.out = ws.act;
+  g1.tiles = ws.tiles;
+  g1.N = 2 * I;
+  g1.K = H;
+  g1.n_col_tiles = cdiv(2 * I, 256);
+  g1.limit = w->swiglu_limit;
+  rc = run_gemm(g1, true, EPI_SWIGLU, rpt, max_tiles, s);
+  if (rc != GPTOSS_OK) return rc;
+
+  GemmParams g2{};
+  g2.A = ws.act;
+  g2.W = (const bf16_t *)w->w2;
+  g2.bias = w->b2;
+  g2.out = ws.y2;
+  g2.tiles = ws.tiles;
+  g2.N = H;
+  g2.K = I;
+  g2.n_col_tiles = cdiv(H, 256);
+  rc = run_gemm(g2, false, EPI_F32, rpt, max_tiles, s);
+  if (rc != GPTOSS_OK) return rc;
+
+  return run_combine(ws.y2, ws.topk_w, ws.inv_perm, out, B, H, k, accumulate, s);
+}

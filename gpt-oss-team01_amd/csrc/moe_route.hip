@@ -1,0 +1,296 @@
+// MoE routing for gfx950: router GEMM (bf16 MFMA 16x16x32), top-k + softmax gating with wave
+// shuffles, and a stable counting sort of the (token,slot) pairs by expert built from wave
+// ballots and an LDS histogram (no global atomics), which also emits the tile list that the
+// grouped GEMMs schedule from.
+#include "common.hpp"
+
+namespace gptoss {
+
+// ------------------------------------------------------------------------------------------------
+// Router GEMM: logits[B,E] = t[B,H] . Wr[E,H]^T + br.  One workgroup = 16 token rows x all experts;
+// its 4 waves split the K loop (k-steps of 32 interleaved) and reduce through LDS.
+// ------------------------------------------------------------------------------------------------
+template <int NB>  // number of 16-expert column blocks held per wave
+__global__ __launch_bounds__(256) void router_gemm_kernel(const bf16_t *__restrict__ t,
+                                                          const bf16_t *__restrict__ wr,
+                                                          const float *__restrict__ br,
+                                                          float *__restrict__ logits, int B, int H,
+                                                          int E) {
+  __shared__ float red[3][16][NB * 16 + 1];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r0 = blockIdx.x * 16;
+  const int arow = min(r0 + (lane & 15), B - 1);
+  const int kq = (lane >> 4) * 8;
+  const bf16_t *ap = t + (size_t)arow * H + kq;
+  f32x4 acc[NB];
+#pragma unroll
+  for (int nb = 0; nb < NB; nb++) acc[nb] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int ksteps = H / 32;
+  for (int ks = wave; ks < ksteps; ks += 4) {
+    u32x4 a = *reinterpret_cast<const u32x4 *>(ap + ks * 32);
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++) {
+      int e = nb * 16 + (lane & 15);
+      u32x4 b = u32x4{0u, 0u, 0u, 0u};
+      if (e < E) b = *reinterpret_cast<const u32x4 *>(wr + (size_t)e * H + ks * 32 + kq);
+      acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a), as_bf16x8(b), acc[nb], 0, 0, 0);
+    }
+  }
+  if (wave > 0) {
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+      for (int i = 0; i < 4; i++)
+        red[wave - 1][(lane >> 4) * 4 + i][nb * 16 + (lane & 15)] = acc[nb][i];
+  }
+  __syncthreads();
+  if (wave == 0) {
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++) {
+      int e = nb * 16 + (lane & 15);
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        int r = (lane >> 4) * 4 + i;
+        if (e < E && r0 + r < B) {
+          float v = acc[nb][i] + red[0][r][e] + red[1][r][e] + red[2][r][e];
+          if (br) v += br[e];
+          logits[(size_t)(r0 + r) * E + e] = v;
+        }
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Top-k + softmax.  32 lanes per token (two tokens per wave); lane j holds experts j, j+32, ...
+// Selection = k rounds of (local best, 5-step butterfly) ordered by (value desc, expert id asc).
+// ------------------------------------------------------------------------------------------------
+template <int NJ>
+__global__ __launch_bounds__(256) void topk_softmax_kernel(const float *__restrict__ logits, int B,
+                                                           int E, int k, float *__restrict__ topk_w,
+                                                           int *__restrict__ topk_i) {
+  const int sub = threadIdx.x & 31;
+  const int token = (blockIdx.x * 256 + threadIdx.x) >> 5;
+  const bool live = token < B;
+  const float *row = logits + (size_t)(live ? token : 0) * E;
+  float v[NJ];
+#pragma unroll
+  for (int j = 0; j < NJ; j++) {
+    int e = sub + 32 * j;
+    v[j] = (live && e < E) ? row[e] : -INFINITY;
+  }
+  uint32_t used = 0;
+  float pick_v[8];
+  int pick_i[8];
+  constexpr int NONE = 0x7fffffff;
+#pragma unroll
+  for (int s = 0; s < 8; s++) {
+    pick_v[s] = -INFINITY;
+    pick_i[s] = 0;
+    if (s < k) {
+      float bv = -INFINITY;
+      int bi = NONE;
+#pragma unroll
+      for (int j = 0; j < NJ; j++) {
+        int e = sub + 32 * j;
+        bool ok = !((used >> j) & 1u) && e < E;
+        if (ok && (bi == NONE || v[j] > bv || (v[j] == bv && e < bi))) {
+          bv = v[j];
+          bi = e;
+        }
+      }
+#pragma unroll
+      for (int m = 16; m >= 1; m >>= 1) {
+        float ov = __shfl_xor(bv, m, 64);
+        int oi = __shfl_xor(bi, m, 64);
+        if (oi != NONE && (bi == NONE || ov > bv || (ov == bv && oi < bi))) {
+          bv = ov;
+          bi = oi;
+        }
+      }
+      if (bi != NONE && (bi & 31) == sub) used |= 1u << (bi >> 5);
+      pick_v[s] = bv;
+      pick_i[s] = bi;
+    }
+  }
+  if (live && sub == 0) {
+    // softmax over the k picked values: exp in float, sum and divide in double (run.cpp:319-337)
+    float ex[8];
+    double sum = 0.0;
+#pragma unroll
+    for (int s = 0; s < 8; s++) {
+      ex[s] = (s < k) ? expf(pick_v[s] - pick_v[0]) : 0.f;
+      sum += ex[s];
+    }
+#pragma unroll
+    for (int s = 0; s < 8; s++) {
+      if (s < k) {
+        topk_w[(size_t)token * k + s] = (float)((double)ex[s] / sum);
+        topk_i[(size_t)token * k + s] = pick_i[s];
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Stable counting sort of P = B*k pairs by expert in ONE workgroup of 1024 threads (16 waves).
+// Each wave owns a contiguous range of pairs.  Inside a 64-pair step the lanes holding the same
+// expert are found with log2(E) ballots; the lowest such lane adds their count to the wave's own
+// LDS histogram row, so no atomics are needed and the order is the pair order (stable).
+// ------------------------------------------------------------------------------------------------
+constexpr int SORT_THREADS = 1024;
+constexpr int SORT_WAVES = SORT_THREADS / 64;
+
+__device__ __forceinline__ uint64_t same_expert_mask(int e, bool valid, int nbits) {
+  uint64_t mask = __ballot(valid);
+  for (int b = 0; b < nbits; b++) {
+    bool bit = (e >> b) & 1;
+    uint64_t bal = __ballot(valid && bit);
+    mask &= bit ? bal : ~bal;
+  }
+  return mask;
+}
+
+__global__ __launch_bounds__(SORT_THREADS) void group_sort_kernel(
+    const int *__restrict__ topk_i, int P, int E, int nbits, int *__restrict__ expert_offsets,
+    int *__restrict__ sorted_pair_ids, int *__restrict__ inv_perm, int *__restrict__ tiles,
+    int rows_per_tile) {
+  extern __shared__ int smem[];
+  int *hist = smem;                    // [SORT_WAVES][E] per-wave counts, then per-wave cursors
+  int *total = hist + SORT_WAVES * E;  // [E]
+  int *offs = total + E;               // [E+1]
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const uint64_t lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+
+  for (int i = threadIdx.x; i < SORT_WAVES * E; i += SORT_THREADS) hist[i] = 0;
+  __syncthreads();
+
+  const int steps_total = (P + 63) / 64;
+  const int steps_per_wave = (steps_total + SORT_WAVES - 1) / SORT_WAVES;
+  const int p_begin = wave * steps_per_wave * 64;
+  const int p_end = min(P, p_begin + steps_per_wave * 64);
+  int *myhist = hist + wave * E;
+
+  for (int p0 = p_begin; p0 < p_end; p0 += 64) {
+    int p = p0 + lane;
+    int e = (p < p_end) ? topk_i[p] : -1;
+    bool valid = (e >= 0 && e < E);
+    uint64_t mask = same_expert_mask(e, valid, nbits);
+    if (valid && (mask & lt_mask) == 0) myhist[e] += __popcll(mask);
+  }
+  __syncthreads();
+
+  // per expert: exclusive prefix over waves (turns counts into in-expert start ranks), and totals
+  for (int e = threadIdx.x; e < E; e += SORT_THREADS) {
+    int run = 0;
+    for (int w = 0; w < SORT_WAVES; w++) {
+      int c = hist[w * E + e];
+      hist[w * E + e] = run;
+      run += c;
+    }
+    total[e] = run;
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e <= E; e += SORT_THREADS) {
+    int o = 0;
+    for (int j = 0; j < e; j++) o += total[j];
+    offs[e] = o;
+    expert_offsets[e] = o;
+  }
+  __syncthreads();
+
+  if (tiles != nullptr && rows_per_tile > 0) {
+    for (int e = threadIdx.x; e < E; e += SORT_THREADS) {
+      int start = 0;
+      for (int j = 0; j < e; j++) start += (total[j] + rows_per_tile - 1) / rows_per_tile;
+      int rows = total[e];
+      int nt = (rows + rows_per_tile - 1) / rows_per_tile;
+      for (int i = 0; i < nt; i++) {
+        int *tp = tiles + 1 + 3 * (start + i);
+        tp[0] = e;
+        tp[1] = offs[e] + i * rows_per_tile;
+        tp[2] = min(rows_per_tile, rows - i * rows_per_tile);
+      }
+      if (e == E - 1) tiles[0] = start + nt;
+    }
+  }
+
+  for (int p0 = p_begin; p0 < p_end; p0 += 64) {
+    int p = p0 + lane;
+    int e = (p < p_end) ? topk_i[p] : -1;
+    bool valid = (e >= 0 && e < E);
+    uint64_t mask = same_expert_mask(e, valid, nbits);
+    if (valid) {
+      int rank = myhist[e] + __popcll(mask & lt_mask);
+      int dst = offs[e] + rank;
+      sorted_pair_ids[dst] = p;
+      inv_perm[p] = dst;
+    }
+    // all lanes of the wave have read myhist before the leaders update it (wave-ordered LDS ops)
+    if (valid && (mask & lt_mask) == 0) myhist[e] += __popcll(mask);
+  }
+}
+
+}  // namespace gptoss
+
+using namespace gptoss;
+
+extern "C" int gptoss_router_gemm(const void *t, const void *w_router, const float *b_router,
+                                  float *logits, int B, int H, int E, void *stream) {
+  GPTOSS_REQUIRE(t && w_router && logits, GPTOSS_ERR_NULL, "router_gemm: null pointer");
+  GPTOSS_REQUIRE(B >= 0 && H > 0 && H % 32 == 0 && E >= 1 && E <= 256, GPTOSS_ERR_DIM,
+                 "router_gemm: need H %% 32 == 0 and 1 <= E <= 256 (B=%d H=%d E=%d)", B, H, E);
+  GPTOSS_REQUIRE(aligned(t, 16) && aligned(w_router, 16), GPTOSS_ERR_ALIGN,
+                 "router_gemm: t and w_router must be 16-byte aligned");
+  if (B == 0) return GPTOSS_OK;
+  hipStream_t s = (hipStream_t)stream;
+  dim3 grid(cdiv(B, 16)), block(256);
+  const bf16_t *tp = (const bf16_t *)t, *wp = (const bf16_t *)w_router;
+  int nb = cdiv(E, 16);
+  if (nb <= 1) router_gemm_kernel<1><<<grid, block, 0, s>>>(tp, wp, b_router, logits, B, H, E);
+  else if (nb <= 2) router_gemm_kernel<2><<<grid, block, 0, s>>>(tp, wp, b_router, logits, B, H, E);
+  else if (nb <= 4) router_gemm_kernel<4><<<grid, block, 0, s>>>(tp, wp, b_router, logits, B, H, E);
+  else if (nb <= 8) router_gemm_kernel<8><<<grid, block, 0, s>>>(tp, wp, b_router, logits, B, H, E);
+  else router_gemm_kernel<16><<<grid, block, 0, s>>>(tp, wp, b_router, logits, B, H, E);
+  GPTOSS_LAUNCH_CHECK("router_gemm_kernel");
+  return GPTOSS_OK;
+}
+
+extern "C" int gptoss_moe_max_tiles(int B, int k, int E, int rows_per_tile) {
+  if (rows_per_tile <= 0 || B < 0 || k <= 0 || E <= 0) return 0;
+  long long P = (long long)B * k;
+  return (int)(P / rows_per_tile) + E;
+}
+
+extern "C" int gptoss_moe_route(const float *logits, int B, int E, int k, float *topk_w,
+                                int *topk_i, int *expert_offsets, int *sorted_pair_ids,
+                                int *inv_perm, int *tiles, int rows_per_tile, void *stream) {
+  GPTOSS_REQUIRE(expert_offsets, GPTOSS_ERR_NULL, "moe_route: null pointer");
+  GPTOSS_REQUIRE(B <= 0 || (logits && topk_w && topk_i && sorted_pair_ids && inv_perm),
+                 GPTOSS_ERR_NULL, "moe_route: null pointer");
+  GPTOSS_REQUIRE(E >= 1 && E <= 256 && k >= 1 && k <= 8 && k <= E && B >= 0, GPTOSS_ERR_DIM,
+                 "moe_route: need 1 <= k <= min(8,E), E <= 256 (B=%d E=%d k=%d)", B, E, k);
+  GPTOSS_REQUIRE((long long)B * k < (1ll << 30), GPTOSS_ERR_DIM, "moe_route: B*k too large");
+  bool tile_ok = rows_per_tile == 0 || rows_per_tile == 32 || rows_per_tile == 64 ||
+                 rows_per_tile == 128 || rows_per_tile == 256;
+  GPTOSS_REQUIRE(tile_ok, GPTOSS_ERR_DIM, "moe_route: rows_per_tile must be 0,32,64,128 or 256");
+  GPTOSS_REQUIRE(rows_per_tile == 0 || tiles, GPTOSS_ERR_NULL, "moe_route: tiles is NULL");
+  hipStream_t s = (hipStream_t)stream;
+  if (B > 0) {
+    dim3 grid(cdiv(B * 32, 256)), block(256);
+    int nj = cdiv(E, 32);
+    if (nj <= 1) topk_softmax_kernel<1><<<grid, block, 0, s>>>(logits, B, E, k, topk_w, topk_i);
+    else if (nj <= 2) topk_softmax_kernel<2><<<grid, block, 0, s>>>(logits, B, E, k, topk_w, topk_i);
+    else if (nj <= 4) topk_softmax_kernel<4><<<grid, block, 0, s>>>(logits, B, E, k, topk_w, topk_i);
+    else topk_softmax_kernel<8><<<grid, block, 0, s>>>(logits, B, E, k, topk_w, topk_i);
+    GPTOSS_LAUNCH_CHECK("topk_softmax_kernel");
+  }
+  int nbits = 0;
+  while ((1 << nbits) < E) nbits++;
+  size_t smem = sizeof(int) * ((size_t)SORT_WAVES * E + E + (E + 1));
+  group_sort_kernel<<<1, SORT_THREADS, smem, s>>>(topk_i, B * k, E, nbits, expert_offsets,
+                                                  sorted_pair_ids, inv_perm,
+                                                  rows_per_tile ? tiles : nullptr, rows_per_tile);
+  GPTOSS_LAUNCH_CHECK("group_sort_kernel");
+  return GPTOSS_OK;
+}

@@ -1,0 +1,131 @@
+"""Thin Python front end over the C ABI for tests and benchmarks.
+
+PyTorch is used only to own device memory and streams; every computation below is a call into
+``libgptoss_mi355.so`` with raw device pointers.  Function names follow the reference's op layer
+(``getp-csrc/include/layer_hip_batch.hpp``, ``kernel.hpp``, ``flash_attn_hip.hpp``)."""
+from __future__ import annotations
+
+import ctypes as C
+
+import torch
+
+from . import lib as _l
+
+
+def _ptr(t):
+    return C.c_void_p(t.data_ptr()) if t is not None else C.c_void_p(0)
+
+
+def _stream():
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _need_gpu():
+    if not torch.cuda.is_available():
+        raise RuntimeError("gptoss_mi355 needs a GPU: there is no CPU path")
+
+
+def pack_weight(w: torch.Tensor, glu: bool = False) -> torch.Tensor:
+    """w: [n_mat, n_out, n_in] (or 2-D) bf16/fp32 on the GPU -> packed bf16 tensor (flat)."""
+    _need_gpu()
+    L = _l.load()
+    if w.dim() == 2:
+        w = w.unsqueeze(0)
+    w = w.contiguous()
+    n_mat, n_out, n_in = w.shape
+    flags = (_l.PACK_GLU if glu else 0)
+    if w.dtype == torch.float32:
+        flags |= _l.PACK_SRC_FP32
+    elif w.dtype != torch.bfloat16:
+        raise TypeError("pack_weight: bf16 or fp32 expected")
+    out = torch.empty(n_mat * n_out * n_in, dtype=torch.bfloat16, device=w.device)
+    _l.check(L.gptoss_pack_weight(_ptr(w), _ptr(out), n_mat, n_out, n_in, flags, _stream()))
+    return out
+
+
+def router_gemm(t, w_router, b_router):
+    _need_gpu()
+    L = _l.load()
+    B, H = t.shape
+    E = w_router.shape[0]
+    logits = torch.empty(B, E, dtype=torch.float32, device=t.device)
+    _l.check(L.gptoss_router_gemm(_ptr(t), _ptr(w_router), _ptr(b_router), _ptr(logits), B, H, E,
+                                  _stream()))
+    return logits
+
+
+def moe_route(logits, k, rows_per_tile=0):
+    """-> topk_w [B,k], topk_i [B,k], expert_offsets [E+1], sorted_pair_ids [B*k], inv_perm [B*k],
+    tiles (or None)."""
+    _need_gpu()
+    L = _l.load()
+    B, E = logits.shape
+    dev = logits.device
+    topk_w = torch.empty(B, k, dtype=torch.float32, device=dev)
+    topk_i = torch.empty(B, k, dtype=torch.int32, device=dev)
+    off = torch.empty(E + 1, dtype=torch.int32, device=dev)
+    srt = torch.full((B * k,), -1, dtype=torch.int32, device=dev)
+    inv = torch.full((B * k,), -1, dtype=torch.int32, device=dev)
+    tiles = None
+    if rows_per_tile:
+        n = L.gptoss_moe_max_tiles(B, k, E, rows_per_tile)
+        tiles = torch.full((1 + 3 * n,), -1, dtype=torch.int32, device=dev)
+    _l.check(L.gptoss_moe_route(_ptr(logits), B, E, k, _ptr(topk_w), _ptr(topk_i), _ptr(off),
+                                _ptr(srt), _ptr(inv), _ptr(tiles), rows_per_tile, _stream()))
+    return topk_w, topk_i, off, srt, inv, tiles
+
+
+class MoeLayer:
+    """Device weights of one MoE block in the layout the kernels read, plus a workspace."""
+
+    def __init__(self, w_router, b_router, w1, b1, w2, b2, top_k=4, swiglu_limit=7.0,
+                 max_tokens=1024):
+        _need_gpu()
+        self.L = _l.load()
+        E, H = w_router.shape
+        I = w2.shape[2]
+        assert tuple(w1.shape) == (E, 2 * I, H) and tuple(w2.shape) == (E, H, I)
+        self.E, self.H, self.I, self.k = E, H, I, top_k
+        dev = w_router.device
+        self.w_router = w_router.to(torch.bfloat16).contiguous()
+        self.b_router = b_router.to(torch.float32).contiguous()
+        self.w1 = pack_weight(w1, glu=True)
+        self.b1 = b1.to(torch.float32).contiguous()
+        self.w2 = pack_weight(w2)
+        self.b2 = b2.to(torch.float32).contiguous()
+        self.desc = _l.MoeWeights(E, top_k, H, I, swiglu_limit, self.w_router.data_ptr(),
+                                  self.b_router.data_ptr(), self.w1.data_ptr(),
+                                  self.b1.data_ptr(), self.w2.data_ptr(), self.b2.data_ptr())
+        self.max_tokens = max_tokens
+        self.ws_bytes = self.L.gptoss_moe_workspace_bytes(max_tokens, E, top_k, H, I)
+        self.ws = torch.empty(self.ws_bytes, dtype=torch.uint8, device=dev)
+        self._last_B = 0
+
+    def forward(self, t, out=None, accumulate=False):
+        B = t.shape[0]
+        assert B <= self.max_tokens and t.dtype == torch.bfloat16 and t.is_contiguous()
+        if out is None:
+            out = torch.empty(B, self.H, dtype=torch.float32, device=t.device)
+        _l.check(self.L.gptoss_moe_forward(C.byref(self.desc), _ptr(t), B, _ptr(out),
+                                           1 if accumulate else 0, _ptr(self.ws), self.ws_bytes,
+                                           _stream()))
+        self._last_B = B
+        return out
+
+    def routing_views(self):
+        """Routing results of the last forward call as torch tensors (copies)."""
+        B, E, k = self._last_B, self.E, self.k
+        ptrs = [C.c_void_p() for _ in range(6)]
+        _l.check(self.L.gptoss_moe_workspace_views(_ptr(self.ws), B, E, k, self.H, self.I,
+                                                   *[C.byref(p) for p in ptrs]))
+        base = self.ws.data_ptr()
+        shapes = [((B, E), torch.float32), ((B, k), torch.float32), ((B, k), torch.int32),
+                  ((E + 1,), torch.int32), ((B * k,), torch.int32), ((B * k,), torch.int32)]
+        out = []
+        for p, (shape, dt) in zip(ptrs, shapes):
+            off = p.value - base
+            n = 1
+            for s in shape:
+                n *= s
+            out.append(self.ws[off:off + n * 4].view(dt).view(shape).clone())
+        return out

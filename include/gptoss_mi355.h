@@ -1,0 +1,220 @@
+/*
+ * gptoss_mi355 -- C ABI of the MI355X (gfx950) GPT-OSS decode hot path.
+ *
+ * This is the boundary the reference's host code binds instead of the C++ op layer in
+ * getp-csrc/include/{layer_hip_batch,kernel,flash_attn_hip}.hpp.  Conventions, all entry points:
+ *   - plain pointers and sizes only; every data pointer is DEVICE memory unless its name starts
+ *     with host_;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream); calls enqueue work
+ *     and return without synchronising, never allocate, and never abort;
+ *   - return value: GPTOSS_OK or an error code; gptoss_last_error_string() gives the text of the
+ *     calling thread's last error;
+ *   - scratch memory comes from the caller: ask gptoss_*_workspace_bytes, pass a 256-byte aligned
+ *     device buffer of at least that size.  One workspace may be reused by consecutive calls on
+ *     the same stream; calls sharing a workspace on different streams race;
+ *   - thread-compatible: distinct workspaces/streams may be driven from distinct host threads.
+ *
+ * Weight matrices are [n_out, n_in] with n_in contiguous, exactly as the flat .bin stores them
+ * (reference run.cpp:54-80); the reference instead transposes every matrix to [n_in, n_out] while
+ * loading (getp-csrc/src/alloc.cpp:27-35,112-127).  GEMM entry points take them in the packed
+ * MFMA-fragment order produced by gptoss_pack_weight().
+ */
+#ifndef GPTOSS_MI355_H
+#define GPTOSS_MI355_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+  GPTOSS_OK = 0,
+  GPTOSS_ERR_NULL = 1,      /* a required pointer is NULL */
+  GPTOSS_ERR_DIM = 2,       /* unsupported or inconsistent dimension */
+  GPTOSS_ERR_ALIGN = 3,     /* pointer not aligned as required */
+  GPTOSS_ERR_WORKSPACE = 4, /* workspace missing or too small */
+  GPTOSS_ERR_HIP = 5,       /* HIP runtime / launch error */
+  GPTOSS_ERR_STATE = 6,     /* call not valid in the engine's current state */
+  GPTOSS_ERR_IO = 7         /* checkpoint file problem */
+};
+
+/* Text of the last error raised on the calling thread ("" if none).  No reference counterpart:
+ * the reference prints and aborts (getp-csrc/include/tensor.hpp:20-27). */
+const char *gptoss_last_error_string(void);
+
+/* ABI version of this header (major*100+minor). */
+int gptoss_abi_version(void);
+
+/* ------------------------------------------------------------------ weight layout ---------- */
+
+/* Flags for gptoss_pack_weight. */
+enum {
+  GPTOSS_PACK_SRC_FP32 = 1, /* source elements are fp32 (the .bin payload); default bf16 */
+  GPTOSS_PACK_GLU = 2       /* rows are interleaved (gate,up) pairs (run.cpp:664-667): reorder them
+                               so a wave holds gate and up of the same pair in one lane */
+};
+
+/* Bytes of n_mat packed [n_out,n_in] matrices (bf16). */
+size_t gptoss_packed_weight_bytes(int n_mat, int n_out, int n_in);
+
+/* Repack n_mat row-major [n_out,n_in] matrices (device, bf16 or fp32) into MFMA-fragment order.
+ * Replaces the host-side transposes of getp-csrc/src/alloc.cpp:27-35,52-59,79-88,112-127,155-170.
+ * Needs n_out % 32 == 0 (64 with GPTOSS_PACK_GLU) and n_in % 64 == 0. */
+int gptoss_pack_weight(const void *src, void *dst, int n_mat, int n_out, int n_in, int flags,
+                       void *stream);
+
+/* ------------------------------------------------------------------ MoE routing ------------ */
+
+/* logits[B,E] = t[B,H] . w_router[E,H]^T + b_router[E]     (bf16 x bf16 -> fp32)
+ * Replaces router_gemm_batched_quantize (getp-csrc/src/layer_hip_batch.cpp:1006-1044).
+ * t bf16 [B,H]; w_router bf16 [E,H] row-major (unpacked); b_router fp32 [E] or NULL.
+ * Needs H % 32 == 0, E % 16 == 0, E <= 256. */
+int gptoss_router_gemm(const void *t, const void *w_router, const float *b_router, float *logits,
+                       int B, int H, int E, void *stream);
+
+/* Sizes of the routing outputs for B tokens: ints in the tile list. */
+int gptoss_moe_max_tiles(int B, int k, int E, int rows_per_tile);
+
+/* Top-k gating and expert grouping from router logits.  Replaces
+ *   topk_softmax_batched        (layer_hip_batch.cpp:1087-1203): top-k, descending, lowest expert
+ *                               id first among equal logits; softmax over the k picked values;
+ *   moe_build_offsets           (kernel.cpp:504-542,851-865): counting sort of the B*k pairs
+ *                               (pair = token*k + slot) by expert, STABLE (ascending pair id inside
+ *                               an expert);
+ *   moe_get_max_rows_per_expert (kernel.cpp:709-719,916-925): replaced by a device-side tile list,
+ *                               no host read-back.
+ * Outputs (device): topk_w fp32 [B,k], topk_i int32 [B,k], expert_offsets int32 [E+1],
+ * sorted_pair_ids int32 [B*k], inv_perm int32 [B*k] (inv_perm[pair] = its row in the sorted
+ * order), tiles int32 [1 + 3*gptoss_moe_max_tiles()] = {n_tiles, (expert,row0,rows)...} cutting
+ * every expert's rows into tiles of rows_per_tile (may be NULL with rows_per_tile 0).
+ * Needs 1 <= k <= 8, k <= E, E % 32 == 0, E <= 256, rows_per_tile in {0,32,64,128,256}. */
+int gptoss_moe_route(const float *logits, int B, int E, int k, float *topk_w, int *topk_i,
+                     int *expert_offsets, int *sorted_pair_ids, int *inv_perm, int *tiles,
+                     int rows_per_tile, void *stream);
+
+/* ------------------------------------------------------------------ MoE layer -------------- */
+
+typedef struct {
+  int n_experts;         /* E */
+  int top_k;             /* k */
+  int hidden;            /* H */
+  int intermediate;      /* I */
+  float swiglu_limit;    /* clamp, 7.0 */
+  const void *w_router;  /* bf16 [E,H] row-major */
+  const float *b_router; /* fp32 [E] */
+  const void *w1;        /* experts' gate/up matrices [E,2I,H], packed with GPTOSS_PACK_GLU;
+                            for the MXFP4 entry point: gptoss_pack_mxfp4 output */
+  const float *b1;       /* fp32 [E,2I], interleaved (gate,up) as in the .bin */
+  const void *w2;        /* experts' down matrices [E,H,I], packed */
+  const float *b2;       /* fp32 [E,H] */
+} gptoss_moe_weights;
+
+size_t gptoss_moe_workspace_bytes(int B, int E, int k, int H, int I);
+
+/* One MoE block for B tokens:  out[B,H] (+)= sum_slot w[b,slot] * FFN_expert(b,slot)(t[b]).
+ * Replaces the sequence router_gemm_batched_quantize .. moe_scatter_aggregate_hip_120b (+ the
+ * residual add_vector_batched when accumulate != 0) of forward_gpu_20b_batched
+ * (getp-csrc/src/model.cpp:74-131): router GEMM, top-k softmax, stable grouping, grouped GEMM1
+ * with the token gather folded into its operand load and clamped SwiGLU folded into its epilogue
+ * (kernel.cpp:560-573,636-685,927-952), grouped GEMM2 (kernel.cpp:1061-1089) and a deterministic
+ * per-token weighted combine in slot order (replaces the atomicAdd scatter, kernel.cpp:748-768).
+ * t bf16 [B,H]; out fp32 [B,H].  Needs H % 64 == 0, I % 64 == 0, E % 32 == 0, E <= 256, k <= 8. */
+int gptoss_moe_forward(const gptoss_moe_weights *w, const void *t, int B, float *out,
+                       int accumulate, void *workspace, size_t workspace_bytes, void *stream);
+
+/* Views into a workspace after gptoss_moe_forward (for tests and tracing): device pointers to
+ * logits fp32 [B,E], topk_w [B,k], topk_i [B,k], expert_offsets [E+1], sorted_pair_ids [B*k],
+ * inv_perm [B*k].  Any output pointer may be NULL. */
+int gptoss_moe_workspace_views(void *workspace, int B, int E, int k, int H, int I, float **logits,
+                               float **topk_w, int **topk_i, int **expert_offsets,
+                               int **sorted_pair_ids, int **inv_perm);
+
+/* MXFP4 expert weights (OCP MX: e2m1 codes, low nibble = even element, one e8m0 scale per 32
+ * elements along n_in; format of export_model_bin/gpt-oss-20b/export_model_bin.py:66-123).  The
+ * reference dequantises offline to bf16 and has no FP4 kernel. */
+size_t gptoss_packed_mxfp4_bytes(int n_mat, int n_out, int n_in);
+/* blocks uint8 [n_mat,n_out,n_in/2], scales uint8 [n_mat,n_out,n_in/32] -> packed. */
+int gptoss_pack_mxfp4(const void *blocks, const void *scales, void *dst, int n_mat, int n_out,
+                      int n_in, int flags, void *stream);
+/* Same contract as gptoss_moe_forward with w->w1 / w->w2 in gptoss_pack_mxfp4 order. */
+int gptoss_moe_forward_mxfp4(const gptoss_moe_weights *w, const void *t, int B, float *out,
+                             int accumulate, void *workspace, size_t workspace_bytes,
+                             void *stream);
+
+/* ------------------------------------------------------------------ decode attention ------- */
+
+/* The KV cache layout is internal (tiled for 128-bit streaming and MFMA operand order); size it
+ * with gptoss_kv_cache_bytes and fill it with gptoss_kv_cache_write.  `capacity` = token slots per
+ * sequence (multiple of 64); position p lives in slot p % capacity, so a cache with capacity ==
+ * window is the ring buffer the reference keeps for its sliding-window layers
+ * (getp-csrc/src/alloc.cpp:245-250). */
+size_t gptoss_kv_cache_bytes(int B, int n_kv, int head_dim, int capacity); /* for K or V alone */
+
+/* Store n_tok consecutive positions [pos0, pos0+n_tok) of every sequence.  k_rows/v_rows bf16
+ * [B, n_tok, n_kv, head_dim] (K already rotated).  Bulk form of the cache write in
+ * qkv_split_rope_store_kernel (layer_hip_batch.cpp:686-776). */
+int gptoss_kv_cache_write(void *k_cache, void *v_cache, const void *k_rows, const void *v_rows,
+                          int B, int n_kv, int head_dim, int capacity, int pos0, int n_tok,
+                          void *stream);
+
+size_t gptoss_attn_workspace_bytes(int B, int n_q, int n_kv, int head_dim, int max_len);
+
+/* Single-query attention with sinks and optional sliding window over the bf16 KV cache.
+ * Replaces single_query_attn_flash_batched_quantize (getp-csrc/src/flash_attn_hip.cpp:847-923).
+ *   q fp32 [B,n_q,D] (rotated); lens int32 [B] = cached positions per sequence (pos+1; the
+ *   reference has one scalar pos for the whole batch); window > 0 keeps the last `window`
+ *   positions; sinks fp32 [n_q] or NULL; out bf16 [B,n_q,D].
+ *   max_len: upper bound of lens known to the host (sizes the split of long sequences).
+ * Needs D in {32,64}, n_q % n_kv == 0, n_q/n_kv <= 16. */
+int gptoss_attn_decode(const float *q, const void *k_cache, const void *v_cache, const int *lens,
+                       const float *sinks, void *out, int B, int n_q, int n_kv, int head_dim,
+                       int capacity, int window, int max_len, void *workspace,
+                       size_t workspace_bytes, void *stream);
+
+/* ------------------------------------------------------------------ engine ------------------ */
+
+/* The 60-byte header of the flat .bin (reference run.cpp:25-45), same field order. */
+typedef struct {
+  int vocab_size, hidden_dim, n_experts, experts_per_token, intermediate_dim, n_layers;
+  int head_dim, n_attn_heads, n_kv_heads, seq_len, initial_context_length;
+  float rope_theta, rope_scaling_factor;
+  int sliding_window;
+  float swiglu_limit;
+} gptoss_config;
+
+typedef struct gptoss_engine gptoss_engine;
+
+enum {
+  GPTOSS_ENGINE_SYNTHETIC = 1, /* host_weights ignored: N(0,0.02) bf16 weights generated on device */
+  GPTOSS_ENGINE_PRECISE = 2    /* keep activations at fp32 accuracy in every GEMM (3-term bf16
+                                  split) instead of the reference GPU path's bf16 staging */
+};
+
+/* Build device weights (bf16, packed) and run state for up to max_batch sequences of up to
+ * max_seq positions.  host_weights = the fp32 payload of the .bin just past the header (host
+ * memory, e.g. the mmap the reference's build_transformer makes).  Replaces our_init
+ * (getp-csrc/src/alloc.cpp:1035-1073) for one GPU.  This call allocates and synchronises. */
+int gptoss_engine_create(const gptoss_config *cfg, const float *host_weights, int max_batch,
+                         int max_seq, int flags, uint64_t seed, gptoss_engine **out);
+
+/* One lock-step decode step: feed host_tokens[B] at position pos, return the arg-max next ids
+ * (lowest id wins ties) in host_next[B].  Replaces forward_gpu_20b_batched
+ * (getp-csrc/src/model.cpp:6-151).  Synchronises once, to hand the ids back. */
+int gptoss_engine_step(gptoss_engine *e, const int *host_tokens, int pos, int B, int *host_next);
+
+/* Greedy generation with the reference's getp loop semantics
+ * (getp-csrc/submit/getp_run_submit.cpp:60-96): prompts int32 [n_req, prompt_stride] with
+ * n_prompt[r] ids each; out int32 [n_req, max_seq_len+1], terminated by -1; returns the harness's
+ * generated-token count in *n_generated. */
+int gptoss_engine_generate(gptoss_engine *e, const int *host_prompts, const int *host_n_prompt,
+                           int prompt_stride, int n_req, int max_seq_len, int *host_out,
+                           long long *n_generated);
+
+void gptoss_engine_destroy(gptoss_engine *e);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* GPTOSS_MI355_H */
