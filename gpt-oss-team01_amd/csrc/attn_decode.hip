@@ -1,0 +1,423 @@
+// Single-query (decode) attention over a bf16 KV cache for gfx950, with attention sinks, optional
+// sliding window, per-sequence lengths and grouped-query sharing.
+//
+// The op is bound by streaming K and V once from HBM, so:
+//   * one wave owns one (sequence, kv head, chunk of the context) and serves ALL query heads of
+//     that kv head from a single pass over K and V (the reference re-reads KV once per q head);
+//   * scores and outputs are computed on the matrix cores in transposed form so the softmax
+//     probabilities leave the first MFMA already in the operand layout of the second one:
+//         S^T[token, head] = K[token, :] . Q^T[:, head]        (v_mfma_f32_16x16x32_bf16)
+//         O^T[d, head]    += V^T[d, token] . P^T[token, head]
+//     q and p are split into bf16 hi+lo parts (two MFMAs each) so they keep ~16 mantissa bits;
+//   * K is stored [sequence, kv head, slot, d]: a wave reads 16 slots x 128 B = 2 KB contiguous
+//     per 128-bit load pair; V is stored in 32-slot blocks already in V^T operand order, 1 KB
+//     contiguous per load; position p lives in slot p % capacity (ring buffer for window layers);
+//   * long contexts are cut into chunks (flash-decoding): partial (max, sum, O) per chunk, merged
+//     with the sink by a small second kernel; sequences that fit one chunk finish in the first.
+#include <type_traits>
+
+#include "common.hpp"
+
+namespace gptoss {
+
+constexpr int ATT_BLOCK = 64;   // slots per inner iteration
+constexpr float NEG_BIG = -1.0e30f;
+
+struct AttnParams {
+  const float *q;      // [B, n_q, D]
+  const bf16_t *kc;    // [B, n_kv, cap, D]
+  const bf16_t *vc;    // [B, n_kv, cap/32, D/16, 64, 8]
+  const int *lens;     // [B]
+  const float *sinks;  // [n_q] or nullptr
+  bf16_t *out;         // [B, n_q, D]
+  float *part_o;       // [B, max_chunks, n_q, D]
+  float *part_ml;      // [B, max_chunks, n_q, 2]
+  int B, n_q, n_kv, G, cap, window, chunk, max_chunks, max_len;
+  float scale_log2e;   // log2(e) / sqrt(D)
+};
+
+struct SeqRange {
+  int s_begin, s_end;  // slot range to visit (s_begin is a multiple of 64)
+  int t_lo, len;       // active positions are [t_lo, len)
+  int nchunks;
+};
+
+__device__ __forceinline__ SeqRange seq_range(int len, int cap, int window, int chunk, int max_len) {
+  SeqRange r;
+  len = max(0, min(len, max_len));
+  r.len = len;
+  if (len <= cap) {
+    r.t_lo = (window > 0) ? max(0, len - window) : 0;
+    r.s_begin = r.t_lo & ~(ATT_BLOCK - 1);
+    r.s_end = len;
+  } else {  // ring has wrapped: every slot holds one of the last `cap` positions
+    r.t_lo = (window > 0) ? max(len - window, len - cap) : len - cap;
+    r.s_begin = 0;
+    r.s_end = cap;
+  }
+  r.nchunks = max(1, (r.s_end - r.s_begin + chunk - 1) / chunk);
+  return r;
+}
+
+// position currently stored in slot s (or -1 if the slot has never been written)
+__device__ __forceinline__ int slot_position(int s, int len, int cap) {
+  int d = len - 1 - s;
+  if (d < 0) return -1;
+  return s + (d / cap) * cap;
+}
+
+template <int D>
+__global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
+  constexpr int KS = D / 32;   // k-steps of the score MFMA
+  constexpr int DB = D / 16;   // 16-row blocks of O^T
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int item = blockIdx.x * 4 + wave;
+  const int g = item % p.n_kv;
+  const int rest = item / p.n_kv;
+  const int b = rest % p.B;
+  const int chunk_id = rest / p.B;
+  if (chunk_id >= p.max_chunks) return;
+  const SeqRange r = seq_range(p.lens[b], p.cap, p.window, p.chunk, p.max_len);
+  if (chunk_id >= r.nchunks) return;
+  const int c0 = r.s_begin + chunk_id * p.chunk;
+  const int c1 = min(r.s_end, c0 + p.chunk);
+  const int n = lane & 15, c = lane >> 4;
+  const int G = p.G;
+  const int head = g * G + min(n, G - 1);
+
+  // ---- Q^T operand, split into bf16 hi and lo parts -----------------------------------------
+  bf16x8 qh[KS], ql[KS];
+  {
+    const float *qp = p.q + ((size_t)b * p.n_q + head) * D + c * KS * 8;
+#pragma unroll
+    for (int s = 0; s < KS; s++) {
+      uint32_t h[4], l[4];
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        float x0 = (n < G) ? qp[s * 8 + 2 * j] : 0.f, x1 = (n < G) ? qp[s * 8 + 2 * j + 1] : 0.f;
+        bf16_t h0 = f32_to_bf16(x0), h1 = f32_to_bf16(x1);
+        h[j] = (uint32_t)h0 | ((uint32_t)h1 << 16);
+        l[j] = pack_bf16x2(x0 - bf16_to_f32(h0), x1 - bf16_to_f32(h1));
+      }
+      qh[s] = as_bf16x8(u32x4{h[0], h[1], h[2], h[3]});
+      ql[s] = as_bf16x8(u32x4{l[0], l[1], l[2], l[3]});
+    }
+  }
+
+  const bf16_t *kbase = p.kc + ((size_t)(b * p.n_kv + g) * p.cap) * D;
+  const bf16_t *vbase = p.vc + ((size_t)(b * p.n_kv + g) * p.cap) * D;
+  // lane's K bytes for slot block `blk`: slot blk + tb*16 + n, d chunk c*KS*8 .. +KS*8
+  const size_t k_lane = (size_t)n * D + c * KS * 8;
+  const size_t v_lane = (size_t)lane * 8;
+
+  u32x4 kreg[2][4][KS], vreg[2][2][DB];
+  auto load_kv = [&](int blk, auto buf) {
+    constexpr int R = decltype(buf)::value;
+#pragma unroll
+    for (int tb = 0; tb < 4; tb++)
+#pragma unroll
+      for (int s = 0; s < KS; s++)
+        kreg[R][tb][s] = *reinterpret_cast<const u32x4 *>(kbase + (size_t)(blk + tb * 16) * D + k_lane + s * 8);
+#pragma unroll
+    for (int grp = 0; grp < 2; grp++)
+#pragma unroll
+      for (int db = 0; db < DB; db++)
+        vreg[R][grp][db] = *reinterpret_cast<const u32x4 *>(
+            vbase + ((size_t)((blk >> 5) + grp) * DB + db) * 512 + v_lane);
+  };
+
+  f32x4 o[DB];
+#pragma unroll
+  for (int db = 0; db < DB; db++) o[db] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m_run = NEG_BIG, l_run = 0.f;
+
+  auto process = [&](int blk, auto buf) {
+    constexpr int R = decltype(buf)::value;
+    // scores for 64 slots x 16 head columns
+    f32x4 s4[4];
+#pragma unroll
+    for (int tb = 0; tb < 4; tb++) {
+      f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s = 0; s < KS; s++) {
+        bf16x8 kf = as_bf16x8(kreg[R][tb][s]);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qh[s], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, ql[s], acc, 0, 0, 0);
+      }
+      s4[tb] = acc;
+    }
+    // mask slots outside the active positions (only the edge blocks and wrapped rings need it)
+    const bool edge = (blk < r.t_lo) || (blk + ATT_BLOCK > c1) || (r.len > p.cap);
+    float bmax = NEG_BIG;
+#pragma unroll
+    for (int tb = 0; tb < 4; tb++)
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        float v = s4[tb][i] * p.scale_log2e;
+        if (edge) {
+          int slot = blk + tb * 16 + c * 4 + i;
+          int pos = slot_position(slot, r.len, p.cap);
+          bool ok = slot < c1 && pos >= r.t_lo;
+          v = ok ? v : -INFINITY;
+        }
+        s4[tb][i] = v;
+        bmax = fmaxf(bmax, v);
+      }
+    bmax = fmaxf(bmax, __shfl_xor(bmax, 16, 64));
+    bmax = fmaxf(bmax, __shfl_xor(bmax, 32, 64));
+    const float m_new = fmaxf(m_run, bmax);
+    const float alpha = exp2f(m_run - m_new);
+    m_run = m_new;
+    float psum = 0.f;
+    bf16x8 ph[2], pl[2];
+#pragma unroll
+    for (int grp = 0; grp < 2; grp++) {
+      uint32_t h[4], l[4];
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        // operand k index (c, jj): jj<4 -> slot c*4+jj of the first 16, jj>=4 -> of the second 16
+        float p0 = exp2f(s4[grp * 2 + (j >> 1)][(j & 1) * 2] - m_new);
+        float p1 = exp2f(s4[grp * 2 + (j >> 1)][(j & 1) * 2 + 1] - m_new);
+        psum += p0 + p1;
+        bf16_t h0 = f32_to_bf16(p0), h1 = f32_to_bf16(p1);
+        h[j] = (uint32_t)h0 | ((uint32_t)h1 << 16);
+        l[j] = pack_bf16x2(p0 - bf16_to_f32(h0), p1 - bf16_to_f32(h1));
+      }
+      ph[grp] = as_bf16x8(u32x4{h[0], h[1], h[2], h[3]});
+      pl[grp] = as_bf16x8(u32x4{l[0], l[1], l[2], l[3]});
+    }
+    l_run = l_run * alpha + psum;
+#pragma unroll
+    for (int db = 0; db < DB; db++) {
+#pragma unroll
+      for (int i = 0; i < 4; i++) o[db][i] *= alpha;
+    }
+#pragma unroll
+    for (int grp = 0; grp < 2; grp++)
+#pragma unroll
+      for (int db = 0; db < DB; db++) {
+        u32x4 vv = vreg[R][grp][db];
+        if (edge) {
+          // zero V of inactive slots: never-written cache memory may hold NaN bit patterns
+#pragma unroll
+          for (int w = 0; w < 4; w++) {
+            int s_lo = blk + grp * 32 + (w >> 1) * 16 + c * 4 + (w & 1) * 2;
+            int p_lo = slot_position(s_lo, r.len, p.cap), p_hi = slot_position(s_lo + 1, r.len, p.cap);
+            uint32_t keep = ((s_lo < c1 && p_lo >= r.t_lo) ? 0x0000ffffu : 0u) |
+                            ((s_lo + 1 < c1 && p_hi >= r.t_lo) ? 0xffff0000u : 0u);
+            vv[w] &= keep;
+          }
+        }
+        bf16x8 vf = as_bf16x8(vv);
+        o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, ph[grp], o[db], 0, 0, 0);
+        o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pl[grp], o[db], 0, 0, 0);
+      }
+  };
+
+  using R0 = std::integral_constant<int, 0>;
+  using R1 = std::integral_constant<int, 1>;
+  const int last_blk = max(c0, ((c1 - 1) & ~(ATT_BLOCK - 1)));
+  if (c1 > c0) {
+    load_kv(c0, R0{});
+    int blk = c0;
+    while (true) {
+      load_kv(min(blk + ATT_BLOCK, last_blk), R1{});
+      process(blk, R0{});
+      blk += ATT_BLOCK;
+      if (blk >= c1) break;
+      load_kv(min(blk + ATT_BLOCK, last_blk), R0{});
+      process(blk, R1{});
+      blk += ATT_BLOCK;
+      if (blk >= c1) break;
+    }
+  }
+
+  // ---- per-head totals: sum the partial denominators of the 4 lanes that share a head --------
+  l_run += __shfl_xor(l_run, 16, 64);
+  l_run += __shfl_xor(l_run, 32, 64);
+  if (n >= G) return;
+  const int hq = g * G + n;
+  if (r.nchunks == 1) {
+    float sink2 = p.sinks ? p.sinks[hq] * 1.4426950408889634f : -INFINITY;
+    float M = fmaxf(m_run, sink2);
+    float w = exp2f(m_run - M);
+    float denom = l_run * w + exp2f(sink2 - M);
+    float inv = (denom > 0.f) ? w / denom : 0.f;
+    bf16_t *op = p.out + ((size_t)b * p.n_q + hq) * D;
+#pragma unroll
+    for (int db = 0; db < DB; db++) {
+      u32x2 pk = u32x2{pack_bf16x2(o[db][0] * inv, o[db][1] * inv),
+                       pack_bf16x2(o[db][2] * inv, o[db][3] * inv)};
+      *reinterpret_cast<u32x2 *>(op + db * 16 + c * 4) = pk;
+    }
+  } else {
+    const size_t slot = ((size_t)b * p.max_chunks + chunk_id) * p.n_q + hq;
+    float *po = p.part_o + slot * D;
+#pragma unroll
+    for (int db = 0; db < DB; db++) *reinterpret_cast<f32x4 *>(po + db * 16 + c * 4) = o[db];
+    if (c == 0) {
+      p.part_ml[slot * 2] = m_run;
+      p.part_ml[slot * 2 + 1] = l_run;
+    }
+  }
+}
+
+// Merge the chunk partials of one (sequence, q head) with the sink logit.
+template <int D>
+__global__ __launch_bounds__(256) void attn_reduce_kernel(AttnParams p) {
+  const int pair = blockIdx.x * (256 / D) + threadIdx.x / D;  // (b, head)
+  const int d = threadIdx.x % D;
+  if (pair >= p.B * p.n_q) return;
+  const int b = pair / p.n_q, hq = pair - b * p.n_q;
+  const SeqRange r = seq_range(p.lens[b], p.cap, p.window, p.chunk, p.max_len);
+  if (r.nchunks <= 1) return;  // already finished by the first kernel
+  const float sink2 = p.sinks ? p.sinks[hq] * 1.4426950408889634f : -INFINITY;
+  float M = sink2;
+  for (int ch = 0; ch < r.nchunks; ch++)
+    M = fmaxf(M, p.part_ml[(((size_t)b * p.max_chunks + ch) * p.n_q + hq) * 2]);
+  float denom = exp2f(sink2 - M), acc = 0.f;
+  for (int ch = 0; ch < r.nchunks; ch++) {
+    size_t slot = ((size_t)b * p.max_chunks + ch) * p.n_q + hq;
+    float w = exp2f(p.part_ml[slot * 2] - M);
+    denom += p.part_ml[slot * 2 + 1] * w;
+    acc += p.part_o[slot * D + d] * w;
+  }
+  p.out[((size_t)b * p.n_q + hq) * D + d] = f32_to_bf16(denom > 0.f ? acc / denom : 0.f);
+}
+
+// Bulk cache write: rows [B, n_tok, n_kv, D] -> K [B, n_kv, cap, D], V in 32-slot operand blocks.
+__global__ __launch_bounds__(256) void kv_cache_write_kernel(bf16_t *__restrict__ kc, bf16_t *__restrict__ vc,
+                                                             const bf16_t *__restrict__ k_rows,
+                                                             const bf16_t *__restrict__ v_rows, int B,
+                                                             int n_kv, int D, int cap, int pos0,
+                                                             int n_tok) {
+  const size_t total = (size_t)B * n_tok * n_kv * D;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (size_t)gridDim.x * 256) {
+    int d = (int)(i % D);
+    size_t r = i / D;
+    int g = (int)(r % n_kv);
+    r /= n_kv;
+    int t = (int)(r % n_tok);
+    int b = (int)(r / n_tok);
+    int slot = (pos0 + t) % cap;
+    size_t base = ((size_t)(b * n_kv + g) * cap) * D;
+    kc[base + (size_t)slot * D + d] = k_rows[i];
+    int tt = slot & 31, within = tt & 15;
+    int lane = (within >> 2) * 16 + (d & 15);
+    int j = (tt >> 4) * 4 + (within & 3);
+    vc[base + ((size_t)(slot >> 5) * (D / 16) + (d >> 4)) * 512 + lane * 8 + j] = v_rows[i];
+  }
+}
+
+static int attn_chunk_tokens(int span) { return span > 1024 ? 512 : 256; }
+
+struct AttnPlan {
+  int chunk, max_chunks;
+  size_t part_o_bytes, part_ml_bytes;
+};
+
+static AttnPlan attn_plan(int B, int n_q, int D, int max_len) {
+  AttnPlan pl;
+  pl.chunk = attn_chunk_tokens(max_len);
+  // a window range can start up to 63 slots before its first active position
+  pl.max_chunks = (max_len + ATT_BLOCK - 1 + pl.chunk - 1) / pl.chunk;
+  if (pl.max_chunks < 1) pl.max_chunks = 1;
+  pl.part_o_bytes = align_up((size_t)B * pl.max_chunks * n_q * D * sizeof(float), 256);
+  pl.part_ml_bytes = align_up((size_t)B * pl.max_chunks * n_q * 2 * sizeof(float), 256);
+  return pl;
+}
+
+}  // namespace gptoss
+
+using namespace gptoss;
+
+extern "C" size_t gptoss_kv_cache_bytes(int B, int n_kv, int head_dim, int capacity) {
+  if (B <= 0 || n_kv <= 0 || head_dim <= 0 || capacity <= 0) return 0;
+  return (size_t)B * n_kv * capacity * head_dim * sizeof(bf16_t);
+}
+
+extern "C" int gptoss_kv_cache_write(void *k_cache, void *v_cache, const void *k_rows,
+                                     const void *v_rows, int B, int n_kv, int head_dim,
+                                     int capacity, int pos0, int n_tok, void *stream) {
+  GPTOSS_REQUIRE(k_cache && v_cache && k_rows && v_rows, GPTOSS_ERR_NULL, "kv_cache_write: null pointer");
+  GPTOSS_REQUIRE(B > 0 && n_kv > 0 && (head_dim == 32 || head_dim == 64) && capacity > 0 &&
+                     capacity % 64 == 0 && pos0 >= 0 && n_tok >= 0 && n_tok <= capacity,
+                 GPTOSS_ERR_DIM,
+                 "kv_cache_write: need head_dim in {32,64}, capacity %% 64 == 0, n_tok <= capacity "
+                 "(D=%d capacity=%d n_tok=%d)", head_dim, capacity, n_tok);
+  if (n_tok == 0) return GPTOSS_OK;
+  size_t total = (size_t)B * n_tok * n_kv * head_dim;
+  int grid = (int)((total + 255) / 256 > 65536 ? 65536 : (total + 255) / 256);
+  kv_cache_write_kernel<<<grid, 256, 0, (hipStream_t)stream>>>((bf16_t *)k_cache, (bf16_t *)v_cache,
+                                                               (const bf16_t *)k_rows, (const bf16_t *)v_rows,
+                                                               B, n_kv, head_dim, capacity, pos0, n_tok);
+  GPTOSS_LAUNCH_CHECK("kv_cache_write_kernel");
+  return GPTOSS_OK;
+}
+
+extern "C" size_t gptoss_attn_workspace_bytes(int B, int n_q, int n_kv, int head_dim, int max_len) {
+  if (B <= 0 || n_q <= 0 || n_kv <= 0 || head_dim <= 0 || max_len <= 0) return 0;
+  // sized for the smallest chunk length so that any window/capacity combination fits
+  int max_chunks = (max_len + ATT_BLOCK - 1 + 255) / 256;
+  return align_up((size_t)B * max_chunks * n_q * head_dim * sizeof(float), 256) +
+         align_up((size_t)B * max_chunks * n_q * 2 * sizeof(float), 256);
+}
+
+extern "C" int gptoss_attn_decode(const float *q, const void *k_cache, const void *v_cache,
+                                  const int *lens, const float *sinks, void *out, int B, int n_q,
+                                  int n_kv, int head_dim, int capacity, int window, int max_len,
+                                  void *workspace, size_t workspace_bytes, void *stream) {
+  GPTOSS_REQUIRE(q && k_cache && v_cache && lens && out, GPTOSS_ERR_NULL, "attn_decode: null pointer");
+  GPTOSS_REQUIRE(B > 0 && n_q > 0 && n_kv > 0 && n_q % n_kv == 0 && n_q / n_kv <= 16, GPTOSS_ERR_DIM,
+                 "attn_decode: need n_q %% n_kv == 0 and n_q/n_kv <= 16 (n_q=%d n_kv=%d)", n_q, n_kv);
+  GPTOSS_REQUIRE(head_dim == 32 || head_dim == 64, GPTOSS_ERR_DIM,
+                 "attn_decode: head_dim must be 32 or 64 (got %d)", head_dim);
+  GPTOSS_REQUIRE(capacity > 0 && capacity % 64 == 0 && window >= 0 && max_len > 0, GPTOSS_ERR_DIM,
+                 "attn_decode: need capacity %% 64 == 0, window >= 0, max_len > 0 (capacity=%d)", capacity);
+  GPTOSS_REQUIRE(window == 0 ? max_len <= capacity : window <= capacity, GPTOSS_ERR_DIM,
+                 "attn_decode: the cache must hold every active position (capacity=%d window=%d max_len=%d)",
+                 capacity, window, max_len);
+  GPTOSS_REQUIRE(aligned(q, 16) && aligned(k_cache, 16) && aligned(v_cache, 16) && aligned(out, 8),
+                 GPTOSS_ERR_ALIGN, "attn_decode: pointers must be 16-byte aligned");
+  // longest slot range one sequence can visit: the whole ring once it may have wrapped
+  int span = (max_len > capacity) ? capacity
+                                  : ((window > 0 && window < max_len) ? window : max_len);
+  AttnPlan pl = attn_plan(B, n_q, head_dim, span);
+  GPTOSS_REQUIRE(workspace && aligned(workspace, 256) &&
+                     workspace_bytes >= pl.part_o_bytes + pl.part_ml_bytes,
+                 GPTOSS_ERR_WORKSPACE, "attn_decode: workspace missing, misaligned or smaller than %zu bytes",
+                 pl.part_o_bytes + pl.part_ml_bytes);
+  AttnParams p;
+  p.q = q;
+  p.kc = (const bf16_t *)k_cache;
+  p.vc = (const bf16_t *)v_cache;
+  p.lens = lens;
+  p.sinks = sinks;
+  p.out = (bf16_t *)out;
+  p.part_o = (float *)workspace;
+  p.part_ml = (float *)((unsigned char *)workspace + pl.part_o_bytes);
+  p.B = B;
+  p.n_q = n_q;
+  p.n_kv = n_kv;
+  p.G = n_q / n_kv;
+  p.cap = capacity;
+  p.window = window;
+  p.chunk = pl.chunk;
+  p.max_chunks = pl.max_chunks;
+  p.max_len = max_len;
+  p.scale_log2e = 1.4426950408889634f / sqrtf((float)head_dim);
+  hipStream_t s = (hipStream_t)stream;
+  long long items = (long long)B * n_kv * pl.max_chunks;
+  int grid = (int)((items + 3) / 4);
+  if (head_dim == 64) attn_decode_kernel<64><<<grid, 256, 0, s>>>(p);
+  else attn_decode_kernel<32><<<grid, 256, 0, s>>>(p);
+  GPTOSS_LAUNCH_CHECK("attn_decode_kernel");
+  if (pl.max_chunks > 1) {
+    int per_block = 256 / head_dim;
+    int rgrid = (B * n_q + per_block - 1) / per_block;
+    if (head_dim == 64) attn_reduce_kernel<64><<<rgrid, 256, 0, s>>>(p);
+    else attn_reduce_kernel<32><<<rgrid, 256, 0, s>>>(p);
+    GPTOSS_LAUNCH_CHECK("attn_reduce_kernel");
+  }
+  return GPTOSS_OK;
+}

@@ -31,16 +31,178 @@ constexpr int BK = 64;            // k per LDS slab (4 MFMA k-steps)
 constexpr int LDS_ROW = BK + 8;   // padded row length in bf16 elements (144 B)
 constexpr int BN = 256;           // virtual columns per workgroup (4 waves x 64)
 
+// One (row tile, column tile) work item with a compile-time number of 32-row blocks, so every
+// loop below is fully unrolled and every global load is unconditional (the wait counters the
+// compiler derives stay exact and the prefetches stay in flight across iterations).
 template <int MB, bool GATHER, int EPI>
+__device__ __forceinline__ void gemm_tile(const GemmParams &p, bf16_t *lds, int lds_stage, int mat,
+                                          int row0, int rows, int ct) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int K = p.K, N = p.N;
+  const int n0_raw = ct * BN + wave * 64;
+  const bool wave_active = n0_raw < N;
+  const int n0 = wave_active ? n0_raw : N - 64;  // idle waves of the last column tile redo a valid one
+  const int nslab = K / BK;
+  const int ksteps = K / 16;
+
+  // ---- A: each thread moves one 16-byte chunk per 32-row block and slab -----------------------
+  const int a_row = tid >> 3, a_kc = tid & 7;
+  uint32_t a_off[MB];
+#pragma unroll
+  for (int i = 0; i < MB; i++) {
+    int r = a_row + 32 * i;
+    int src = 0;
+    if (r < rows) {
+      if (GATHER) src = p.row_ids[row0 + r] / p.top_k;
+      else src = row0 + r;
+    } else if (!GATHER) {
+      src = row0;
+    }
+    a_off[i] = (uint32_t)src * (uint32_t)K + a_kc * 8;
+  }
+  u32x4 areg[MB];
+  auto load_a = [&](int s) {
+#pragma unroll
+    for (int i = 0; i < MB; i++) areg[i] = *reinterpret_cast<const u32x4 *>(p.A + a_off[i] + s * BK);
+  };
+  bf16_t *a_dst = lds + a_row * LDS_ROW + a_kc * 8;
+  auto store_a = [&](int stage) {
+#pragma unroll
+    for (int i = 0; i < MB; i++)
+      *reinterpret_cast<u32x4 *>(a_dst + stage * lds_stage + 32 * i * LDS_ROW) = areg[i];
+  };
+
+  // ---- B: two fragment streams per wave, three slabs in the register ring ---------------------
+  const bf16_t *wbase = p.W + (size_t)mat * N * K + ((size_t)(n0 >> 5) * ksteps * 64 + lane) * 8;
+  const size_t frag_stride = (size_t)ksteps * 512;  // elements between adjacent 32-column blocks
+  u32x4 breg[3][2][4];
+  auto load_b = [&](int s, auto ring) {
+    constexpr int R = decltype(ring)::value;
+#pragma unroll
+    for (int f = 0; f < 2; f++)
+#pragma unroll
+      for (int kk = 0; kk < 4; kk++)
+        breg[R][f][kk] = *reinterpret_cast<const u32x4 *>(wbase + f * frag_stride +
+                                                          (size_t)(s * 4 + kk) * 512);
+  };
+
+  f32x16 acc[MB][2];
+#pragma unroll
+  for (int i = 0; i < MB; i++)
+#pragma unroll
+    for (int f = 0; f < 2; f++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[i][f][r] = 0.f;
+
+  const bf16_t *a_src = lds + (lane & 31) * LDS_ROW + (lane >> 5) * 8;
+  auto compute = [&](int stage, auto ring) {
+    constexpr int R = decltype(ring)::value;
+    const bf16_t *base = a_src + stage * lds_stage;
+#pragma unroll
+    for (int kk = 0; kk < 4; kk++) {
+      bf16x8 b0 = as_bf16x8(breg[R][0][kk]), b1 = as_bf16x8(breg[R][1][kk]);
+#pragma unroll
+      for (int i = 0; i < MB; i++) {
+        bf16x8 a = as_bf16x8(*reinterpret_cast<const u32x4 *>(base + i * 32 * LDS_ROW + kk * 16));
+        acc[i][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b0, acc[i][0], 0, 0, 0);
+        acc[i][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b1, acc[i][1], 0, 0, 0);
+      }
+    }
+  };
+
+  using R0 = std::integral_constant<int, 0>;
+  using R1 = std::integral_constant<int, 1>;
+  using R2 = std::integral_constant<int, 2>;
+  const int last = nslab - 1;
+
+  load_b(0, R0{});
+  load_b(min(1, last), R1{});
+  load_a(0);
+  store_a(0);
+  load_a(min(1, last));
+  __syncthreads();
+
+  // slab s: prefetch B and A of slab s+2 (clamped at the end: a harmless re-read), multiply slab
+  // s, publish A of slab s+1 to the other LDS stage.
+  auto body = [&](int s, auto ring, auto ring_next2) {
+    load_b(min(s + 2, last), ring_next2);
+    compute(s & 1, ring);
+    store_a((s + 1) & 1);
+    load_a(min(s + 2, last));
+    __syncthreads();
+  };
+  int s = 0;
+  for (; s + 3 <= nslab; s += 3) {
+    body(s, R0{}, R2{});
+    body(s + 1, R1{}, R0{});
+    body(s + 2, R2{}, R1{});
+  }
+  if (s < nslab) {
+    body(s, R0{}, R2{});
+    if (s + 1 < nslab) body(s + 1, R1{}, R0{});
+  }
+
+  if (!wave_active) return;
+
+  // ---- epilogue ------------------------------------------------------------------------------
+  const int c = lane & 31, rsub = (lane >> 5) * 4;
+  if (EPI == EPI_SWIGLU) {
+    const int half_n = N >> 1;
+    const int j = (n0 >> 1) + c;  // pair index: gate = row 2j, up = row 2j+1 of the .bin matrix
+    float bg = 0.f, bu = 0.f;
+    if (p.bias) {
+      bg = p.bias[(size_t)mat * N + 2 * j];
+      bu = p.bias[(size_t)mat * N + 2 * j + 1];
+    }
+    bf16_t *o = reinterpret_cast<bf16_t *>(p.out);
+    const float L = p.limit;
+#pragma unroll
+    for (int i = 0; i < MB; i++) {
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        int row = i * 32 + (r >> 2) * 8 + rsub + (r & 3);
+        if (row < rows) {
+          float g = acc[i][0][r] + bg, u = acc[i][1][r] + bu;
+          g = fminf(g, L);
+          u = fminf(fmaxf(u, -L), L);
+          float v = g * (1.0f / (1.0f + expf(-1.702f * g)));
+          v *= (u + 1.0f);
+          o[(size_t)(row0 + row) * half_n + j] = f32_to_bf16(v);
+        }
+      }
+    }
+  } else {
+#pragma unroll
+    for (int f = 0; f < 2; f++) {
+      const int col = n0 + f * 32 + c;
+      float bv = p.bias ? p.bias[(size_t)mat * N + col] : 0.f;
+#pragma unroll
+      for (int i = 0; i < MB; i++) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          int row = i * 32 + (r >> 2) * 8 + rsub + (r & 3);
+          if (row < rows) {
+            float v = acc[i][f][r] + bv;
+            if (EPI == EPI_F32)
+              reinterpret_cast<float *>(p.out)[(size_t)(row0 + row) * N + col] = v;
+            else
+              reinterpret_cast<bf16_t *>(p.out)[(size_t)(row0 + row) * N + col] = f32_to_bf16(v);
+          }
+        }
+      }
+    }
+  }
+}
+
+template <int MBMAX, bool GATHER, int EPI>
 __global__ __launch_bounds__(GEMM_THREADS) void grouped_gemm_kernel(GemmParams p) {
-  constexpr int BM = MB * 32;
+  constexpr int BM = MBMAX * 32;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   bf16_t *lds = reinterpret_cast<bf16_t *>(smem_raw);  // [2][BM][LDS_ROW]
   constexpr int STAGE = BM * LDS_ROW;
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-
-  // ---- which (tile, column tile) is this workgroup's ------------------------------------------
+  // ---- which (row tile, column tile) is this workgroup's: workgroups are dealt round-robin to
+  // the 8 XCDs, so XCD x takes the x-th contiguous eighth of the work list -----------------------
   const int n_tiles = p.tiles ? p.tiles[0] : (p.dense_rows + BM - 1) / BM;
   const int total = n_tiles * p.n_col_tiles;
   const int chunk = (total + 7) >> 3;
@@ -60,162 +222,19 @@ __global__ __launch_bounds__(GEMM_THREADS) void grouped_gemm_kernel(GemmParams p
     rows = min(BM, p.dense_rows - row0);
   }
   const int mb = (rows + 31) >> 5;
-  const int K = p.K, N = p.N;
-  const int n0 = ct * BN + wave * 64;
-  const bool wave_active = n0 < N;
-  const int nslab = K / BK;
-  const int ksteps = K / 16;
-
-  // ---- A: each thread moves one 16-byte chunk per 32-row block and slab -----------------------
-  const int a_row = tid >> 3, a_kc = tid & 7;
-  uint32_t a_off[MB];
-#pragma unroll
-  for (int i = 0; i < MB; i++) {
-    int r = a_row + 32 * i;
-    int src = 0;
-    if (r < rows) {
-      if (GATHER) src = p.row_ids[row0 + r] / p.top_k;
-      else src = row0 + r;
-    }
-    a_off[i] = (uint32_t)src * (uint32_t)K + a_kc * 8;
-  }
-  u32x4 areg[MB];
-  auto load_a = [&](int s) {
-#pragma unroll
-    for (int i = 0; i < MB; i++)
-      if (i < mb) areg[i] = *reinterpret_cast<const u32x4 *>(p.A + a_off[i] + s * BK);
-  };
-  auto store_a = [&](int stage) {
-#pragma unroll
-    for (int i = 0; i < MB; i++)
-      if (i < mb)
-        *reinterpret_cast<u32x4 *>(lds + stage * STAGE + (a_row + 32 * i) * LDS_ROW + a_kc * 8) =
-            areg[i];
-  };
-
-  // ---- B: two fragment streams per wave, three slabs in flight --------------------------------
-  const bf16_t *wbase = p.W + (size_t)mat * N * K + ((size_t)(n0 >> 5) * ksteps * 64 + lane) * 8;
-  const size_t frag_stride = (size_t)ksteps * 512;  // elements between adjacent 32-column blocks
-  u32x4 breg[3][2][4];
-  auto load_b = [&](int s, auto ring) {
-    constexpr int R = decltype(ring)::value;
-    if (wave_active) {
-#pragma unroll
-      for (int f = 0; f < 2; f++)
-#pragma unroll
-        for (int kk = 0; kk < 4; kk++)
-          breg[R][f][kk] = *reinterpret_cast<const u32x4 *>(wbase + f * frag_stride +
-                                                            (size_t)(s * 4 + kk) * 512);
-    }
-  };
-
-  f32x16 acc[MB][2];
-#pragma unroll
-  for (int i = 0; i < MB; i++)
-#pragma unroll
-    for (int f = 0; f < 2; f++)
-#pragma unroll
-      for (int r = 0; r < 16; r++) acc[i][f][r] = 0.f;
-
-  const int frag_row = lane & 31, frag_k = (lane >> 5) * 8;
-  auto compute = [&](int stage, auto ring) {
-    constexpr int R = decltype(ring)::value;
-    if (wave_active) {
-      const bf16_t *base = lds + stage * STAGE + frag_row * LDS_ROW + frag_k;
-#pragma unroll
-      for (int kk = 0; kk < 4; kk++) {
-        bf16x8 b0 = as_bf16x8(breg[R][0][kk]), b1 = as_bf16x8(breg[R][1][kk]);
-#pragma unroll
-        for (int i = 0; i < MB; i++) {
-          if (i < mb) {
-            bf16x8 a = as_bf16x8(*reinterpret_cast<const u32x4 *>(base + i * 32 * LDS_ROW + kk * 16));
-            acc[i][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b0, acc[i][0], 0, 0, 0);
-            acc[i][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b1, acc[i][1], 0, 0, 0);
-          }
-        }
-      }
-    }
-  };
-
-  using R0 = std::integral_constant<int, 0>;
-  using R1 = std::integral_constant<int, 1>;
-  using R2 = std::integral_constant<int, 2>;
-
-  load_b(0, R0{});
-  if (nslab > 1) load_b(1, R1{});
-  load_a(0);
-  store_a(0);
-  if (nslab > 1) load_a(1);
-  __syncthreads();
-
-  auto body = [&](int s, auto ring, auto ring_next2) {
-    if (s + 2 < nslab) load_b(s + 2, ring_next2);
-    compute(s & 1, ring);
-    if (s + 1 < nslab) {
-      store_a((s + 1) & 1);
-      if (s + 2 < nslab) load_a(s + 2);
-    }
-    __syncthreads();
-  };
-  for (int s = 0; s < nslab; s += 3) {
-    body(s, R0{}, R2{});
-    if (s + 1 < nslab) body(s + 1, R1{}, R0{});
-    if (s + 2 < nslab) body(s + 2, R2{}, R1{});
-  }
-
-  if (!wave_active) return;
-
-  // ---- epilogue ------------------------------------------------------------------------------
-  const int c = lane & 31, rsub = (lane >> 5) * 4;
-  if (EPI == EPI_SWIGLU) {
-    const int half_n = N >> 1;
-    const int j = (n0 >> 1) + c;  // pair index: gate = row 2j, up = row 2j+1 of the .bin matrix
-    float bg = 0.f, bu = 0.f;
-    if (p.bias) {
-      bg = p.bias[(size_t)mat * N + 2 * j];
-      bu = p.bias[(size_t)mat * N + 2 * j + 1];
-    }
-    bf16_t *o = reinterpret_cast<bf16_t *>(p.out);
-    const float L = p.limit;
-#pragma unroll
-    for (int i = 0; i < MB; i++) {
-      if (i < mb) {
-#pragma unroll
-        for (int r = 0; r < 16; r++) {
-          int row = i * 32 + (r >> 2) * 8 + rsub + (r & 3);
-          if (row < rows) {
-            float g = acc[i][0][r] + bg, u = acc[i][1][r] + bu;
-            g = fminf(g, L);
-            u = fminf(fmaxf(u, -L), L);
-            float v = g * (1.0f / (1.0f + expf(-1.702f * g)));
-            v *= (u + 1.0f);
-            o[(size_t)(row0 + row) * half_n + j] = f32_to_bf16(v);
-          }
-        }
-      }
-    }
+  if (MBMAX >= 8 && mb > 6) {
+    if (mb == 8) gemm_tile<(MBMAX >= 8 ? 8 : MBMAX), GATHER, EPI>(p, lds, STAGE, mat, row0, rows, ct);
+    else gemm_tile<(MBMAX >= 8 ? 7 : MBMAX), GATHER, EPI>(p, lds, STAGE, mat, row0, rows, ct);
+  } else if (MBMAX >= 8 && mb > 4) {
+    if (mb == 6) gemm_tile<(MBMAX >= 8 ? 6 : MBMAX), GATHER, EPI>(p, lds, STAGE, mat, row0, rows, ct);
+    else gemm_tile<(MBMAX >= 8 ? 5 : MBMAX), GATHER, EPI>(p, lds, STAGE, mat, row0, rows, ct);
+  } else if (MBMAX >= 4 && mb > 2) {
+    if (mb == 4) gemm_tile<(MBMAX >= 4 ? 4 : MBMAX), GATHER, EPI>(p, lds, STAGE, mat, row0, rows, ct);
+    else gemm_tile<(MBMAX >= 4 ? 3 : MBMAX), GATHER, EPI>(p, lds, STAGE, mat, row0, rows, ct);
+  } else if (MBMAX >= 2 && mb == 2) {
+    gemm_tile<(MBMAX >= 2 ? 2 : MBMAX), GATHER, EPI>(p, lds, STAGE, mat, row0, rows, ct);
   } else {
-#pragma unroll
-    for (int f = 0; f < 2; f++) {
-      const int col = n0 + f * 32 + c;
-      float bv = p.bias ? p.bias[(size_t)mat * N + col] : 0.f;
-#pragma unroll
-      for (int i = 0; i < MB; i++) {
-        if (i < mb) {
-#pragma unroll
-          for (int r = 0; r < 16; r++) {
-            int row = i * 32 + (r >> 2) * 8 + rsub + (r & 3);
-            if (row < rows) {
-              float v = acc[i][f][r] + bv;
-              if (EPI == EPI_F32)
-                reinterpret_cast<float *>(p.out)[(size_t)(row0 + row) * N + col] = v;
-              else
-                reinterpret_cast<bf16_t *>(p.out)[(size_t)(row0 + row) * N + col] = f32_to_bf16(v);
-            }
-          }
-        }
-      }
-    }
+    gemm_tile<1, GATHER, EPI>(p, lds, STAGE, mat, row0, rows, ct);
   }
 }
 

@@ -79,7 +79,7 @@ SIGNATURES = {
 _lib = None
 
 
-def load(strict: bool = True):
+def load(strict: bool = os.environ.get("GPTOSS_PARTIAL_LIB") != "1"):
     """Load the shared library and bind every declared entry point."""
     global _lib
     if _lib is not None:

@@ -129,3 +129,50 @@ class MoeLayer:
                 n *= s
             out.append(self.ws[off:off + n * 4].view(dt).view(shape).clone())
         return out
+
+
+class KVCache:
+    """bf16 K/V cache of one layer in the kernels' internal layout."""
+
+    def __init__(self, B, n_kv, head_dim, capacity, device="cuda", zero=False):
+        _need_gpu()
+        self.L = _l.load()
+        self.B, self.n_kv, self.D, self.cap = B, n_kv, head_dim, capacity
+        nbytes = self.L.gptoss_kv_cache_bytes(B, n_kv, head_dim, capacity)
+        if nbytes == 0 or capacity % 64:
+            raise ValueError("KVCache: capacity must be a positive multiple of 64")
+        alloc = torch.zeros if zero else torch.empty
+        self.k = alloc(nbytes // 2, dtype=torch.bfloat16, device=device)
+        self.v = alloc(nbytes // 2, dtype=torch.bfloat16, device=device)
+
+    def write(self, k_rows, v_rows, pos0=0):
+        """k_rows, v_rows: bf16 [B, n_tok, n_kv, D] for positions pos0 .. pos0+n_tok-1."""
+        B, n_tok, n_kv, D = k_rows.shape
+        assert (B, n_kv, D) == (self.B, self.n_kv, self.D)
+        assert k_rows.dtype == torch.bfloat16 and v_rows.dtype == torch.bfloat16
+        k_rows, v_rows = k_rows.contiguous(), v_rows.contiguous()
+        _l.check(self.L.gptoss_kv_cache_write(_ptr(self.k), _ptr(self.v), _ptr(k_rows),
+                                              _ptr(v_rows), B, n_kv, D, self.cap, pos0, n_tok,
+                                              _stream()))
+
+
+class AttnDecode:
+    """single_query_attn_flash_batched: q [B,n_q,D] fp32 -> out [B,n_q,D] bf16."""
+
+    def __init__(self, B, n_q, n_kv, head_dim, max_len, device="cuda"):
+        _need_gpu()
+        self.L = _l.load()
+        self.B, self.n_q, self.n_kv, self.D, self.max_len = B, n_q, n_kv, head_dim, max_len
+        self.ws_bytes = self.L.gptoss_attn_workspace_bytes(B, n_q, n_kv, head_dim, max_len)
+        self.ws = torch.empty(max(self.ws_bytes, 256), dtype=torch.uint8, device=device)
+
+    def forward(self, q, cache: KVCache, lens, sinks=None, window=0, out=None, max_len=None):
+        B = q.shape[0]
+        assert q.dtype == torch.float32 and q.is_contiguous() and lens.dtype == torch.int32
+        if out is None:
+            out = torch.empty(B, self.n_q, self.D, dtype=torch.bfloat16, device=q.device)
+        _l.check(self.L.gptoss_attn_decode(_ptr(q), _ptr(cache.k), _ptr(cache.v), _ptr(lens),
+                                           _ptr(sinks), _ptr(out), B, self.n_q, self.n_kv, self.D,
+                                           cache.cap, window, max_len or self.max_len,
+                                           _ptr(self.ws), self.ws_bytes, _stream()))
+        return out

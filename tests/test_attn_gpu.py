@@ -1,0 +1,127 @@
+"""GPU parity of decode attention (sinks, sliding window, GQA, ragged lengths, ring cache)
+against the CPU oracle, through the C ABI."""
+import numpy as np
+import pytest
+import torch
+
+from conftest import TOL_MAX, TOL_MEAN, rel_errors
+
+pytestmark = pytest.mark.gpu
+
+
+def _mk(B, S, n_q, n_kv, D, seed):
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn(B, n_q, D, generator=g)
+    K = torch.randn(B, S, n_kv, D, generator=g).to(torch.bfloat16)
+    V = torch.randn(B, S, n_kv, D, generator=g).to(torch.bfloat16)
+    sinks = torch.randn(n_q, generator=g)
+    return q, K, V, sinks
+
+
+def _run(ops, q, K, V, lens, sinks, window, capacity=None, max_len=None):
+    B, S, n_kv, D = K.shape
+    n_q = q.shape[1]
+    cap = capacity or ((S + 63) // 64 * 64)
+    cache = ops.KVCache(B, n_kv, D, cap)
+    # never-written slots keep whatever the allocator left there, NaN patterns included
+    cache.k.view(torch.int16).fill_(0x7FC1)
+    cache.v.view(torch.int16).fill_(0x7FC1)
+    cache.write(K.cuda(), V.cuda(), 0)
+    attn = ops.AttnDecode(B, n_q, n_kv, D, max_len or int(lens.max()))
+    out = attn.forward(q.cuda(), cache, torch.as_tensor(lens, dtype=torch.int32).cuda(),
+                       None if sinks is None else sinks.cuda(), window=window)
+    torch.cuda.synchronize()
+    return out.float().cpu().numpy()
+
+
+@pytest.mark.parametrize("B,n_q,n_kv,D,lens,window", [
+    (3, 8, 2, 32, [1, 2, 63], 0),                    # tiny-model heads, very short contexts
+    (4, 8, 2, 32, [64, 65, 127, 128], 0),
+    (4, 8, 2, 32, [100, 129, 200, 300], 128),        # window smaller than the context
+    (5, 64, 8, 64, [1, 17, 256, 257, 700], 0),       # 20B heads, one and several chunks
+    (3, 64, 8, 64, [512, 1500, 4096], 0),            # long contexts: 512-token chunks + merge
+    (4, 64, 8, 64, [100, 128, 129, 4000], 128),      # sliding window on a full-length cache
+    (2, 16, 1, 64, [333, 90], 0),                    # 16 query heads per kv head
+    (2, 4, 4, 64, [70, 5], 0),                       # no sharing (MHA)
+])
+def test_attn_matches_oracle(ops, orc, B, n_q, n_kv, D, lens, window):
+    lens = np.asarray(lens, np.int32)
+    S = int(lens.max())
+    q, K, V, sinks = _mk(B, S, n_q, n_kv, D, seed=S + n_q)
+    got = _run(ops, q, K, V, lens, sinks, window)
+    want = orc.attn_decode(q.numpy(), K.float().numpy(), V.float().numpy(), lens, sinks.numpy(), window)
+    assert np.isfinite(got).all()
+    mx, mean = rel_errors(got, want)
+    assert mx <= TOL_MAX and mean <= TOL_MEAN, (mx, mean)
+
+
+def test_attn_no_sink_equals_sdpa(ops):
+    """sinks=None reduces to plain softmax attention (checked against torch SDPA)."""
+    B, n_q, n_kv, D, S = 2, 64, 8, 64, 300
+    q, K, V, _ = _mk(B, S, n_q, n_kv, D, seed=11)
+    lens = np.array([S, S], np.int32)
+    got = _run(ops, q, K, V, lens, None, 0)
+    Kf = K.float().permute(0, 2, 1, 3).repeat_interleave(n_q // n_kv, dim=1)
+    Vf = V.float().permute(0, 2, 1, 3).repeat_interleave(n_q // n_kv, dim=1)
+    want = torch.nn.functional.scaled_dot_product_attention(q.unsqueeze(2), Kf, Vf).squeeze(2).numpy()
+    mx, mean = rel_errors(got, want)
+    assert mx <= TOL_MAX and mean <= TOL_MEAN, (mx, mean)
+
+
+def test_attn_ring_cache_wrapped(ops, orc):
+    """A cache of capacity == window holds position p in slot p % capacity; after wrapping the
+    result equals attention over the last `window` positions."""
+    B, n_q, n_kv, D, W = 3, 8, 2, 32, 128
+    total = [130, 256, 301]
+    S = max(total)
+    q, K, V, sinks = _mk(B, S, n_q, n_kv, D, seed=5)
+    cache = ops.KVCache(B, n_kv, D, W)
+    Kc, Vc = K.cuda(), V.cuda()
+    for p0 in range(0, S, 64):                          # stream the positions through the ring
+        n = min(64, S - p0)
+        cache.write(Kc[:, p0:p0 + n], Vc[:, p0:p0 + n], p0)
+    torch.cuda.synchronize()
+    # sequences shorter than S saw extra writes; rebuild per-sequence caches for exactness
+    outs = []
+    for b in range(B):
+        cb = ops.KVCache(1, n_kv, D, W)
+        for p0 in range(0, total[b], 50):
+            n = min(50, total[b] - p0)
+            cb.write(Kc[b:b + 1, p0:p0 + n], Vc[b:b + 1, p0:p0 + n], p0)
+        attn = ops.AttnDecode(1, n_q, n_kv, D, max_len=2048)
+        o = attn.forward(q[b:b + 1].cuda(), cb, torch.tensor([total[b]], dtype=torch.int32).cuda(),
+                         sinks.cuda(), window=W)
+        outs.append(o.float().cpu().numpy())
+    got = np.concatenate(outs)
+    want = orc.attn_decode(q.numpy(), K.float().numpy(), V.float().numpy(),
+                           np.asarray(total, np.int32), sinks.numpy(), W)
+    mx, mean = rel_errors(got, want)
+    assert mx <= TOL_MAX and mean <= TOL_MEAN, (mx, mean)
+
+
+def test_attn_len1_closed_form(ops):
+    """One cached position: o = v * e^s / (e^s + e^sink)."""
+    B, n_q, n_kv, D = 2, 8, 2, 32
+    q, K, V, sinks = _mk(B, 1, n_q, n_kv, D, seed=3)
+    got = _run(ops, q, K, V, np.array([1, 1], np.int32), sinks, 0)
+    Kf, Vf = K.float().numpy(), V.float().numpy()
+    for b in range(B):
+        for h in range(n_q):
+            g = h // (n_q // n_kv)
+            s = float(q[b, h].numpy() @ Kf[b, 0, g]) / np.sqrt(D)
+            w = np.exp(s) / (np.exp(s) + np.exp(float(sinks[h])))
+            np.testing.assert_allclose(got[b, h], w * Vf[b, 0, g], rtol=1e-2, atol=1e-2)
+
+
+def test_attn_bad_arguments(ops):
+    import ctypes as C
+    from conftest import load_pkg
+    lib = load_pkg("lib")
+    L = lib.load(strict=False)
+    q = torch.zeros(1, 8, 48, device="cuda")
+    rc = L.gptoss_attn_decode(C.c_void_p(q.data_ptr()), C.c_void_p(q.data_ptr()), C.c_void_p(q.data_ptr()),
+                              C.c_void_p(q.data_ptr()), None, C.c_void_p(q.data_ptr()), 1, 8, 2, 48, 64, 0,
+                              10, C.c_void_p(q.data_ptr()), 1 << 20, None)
+    assert rc == 2 and "head_dim" in lib.last_error()
+    rc = L.gptoss_attn_decode(None, None, None, None, None, None, 1, 8, 2, 64, 64, 0, 10, None, 0, None)
+    assert rc == 1
