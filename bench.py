@@ -1,0 +1,220 @@
+#!/usr/bin/env python3
+"""Benchmark of the GPT-OSS decode hot path on one MI355X.
+
+One "step" = one pass of the MoE block (router GEMM, top-4 gating, stable grouping, grouped expert
+GEMMs with clamped SwiGLU, weighted combine) over a batch of 1024 synthetic tokens at the
+GPT-OSS-20B layer shape (hidden 2880, 32 experts, top-4, intermediate 2880), inputs and weights
+resident in HBM.  Successive steps alternate between two independent sets of layer weights
+(2 x 1.6 GB) so no cache level can keep them.
+
+Prints ONE JSON line: the headline MoE-layer tokens/s with its roofline (dominant kernel = the
+fused gather + GEMM1 + SwiGLU kernel, timed with HIP events on its launch stream) and the CPU
+baseline (the CPU oracle restatement of the reference run.cpp MoE loop on a token slice), plus,
+under "extra", the decode-attention HBM rates and the per-kernel breakdown.
+"""
+from __future__ import annotations
+
+import argparse
+import importlib
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0         # MI355X HBM3E
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--tokens", type=int, default=1024)
+    ap.add_argument("--cpu-tokens", type=int, default=1024,
+                    help="token slice timed on the CPU baseline (0 = skip)")
+    ap.add_argument("--no-attn", action="store_true", help="skip the decode-attention figures")
+    ap.add_argument("--no-e2e", action="store_true", help="skip the end-to-end decode figure")
+    return ap.parse_args()
+
+
+def bench_moe(ops, torch, args):
+    B, E, H, I, k = args.tokens, 32, 2880, 2880, 4
+    dev = "cuda"
+    g = torch.Generator(device=dev).manual_seed(1234)
+
+    def n(*shape, std=0.02):
+        return (torch.randn(*shape, device=dev, generator=g) * std).to(torch.bfloat16)
+
+    raw, layers = [], []
+    for _ in range(2):
+        w = dict(w_router=n(E, H), b_router=n(E), w1=n(E, 2 * I, H), b1=n(E, 2 * I),
+                 w2=n(E, H, I), b2=n(E, H))
+        layers.append(ops.MoeLayer(w["w_router"], w["b_router"], w["w1"], w["b1"], w["w2"],
+                                   w["b2"], top_k=k, swiglu_limit=7.0, max_tokens=B))
+        raw.append(w if not raw else None)      # keep one unpacked copy for the CPU baseline
+        if raw[-1] is None:
+            del w
+    t = n(B, H, std=1.0)
+    out = torch.empty(B, H, dtype=torch.float32, device=dev)
+
+    for i in range(args.warmup):
+        layers[i % 2].forward(t, out)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        layers[i % 2].forward(t, out)
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    # same steps again with per-kernel HIP events on the launch stream
+    trace = ops.KernelTrace(capacity=8 * args.steps + 8)
+    with trace:
+        for i in range(args.steps):
+            layers[i % 2].forward(t, out)
+    kern = trace.summary()
+
+    flops = 2.0 * B * k * H * 3 * I + 2.0 * B * H * E
+    w1_bytes = E * 2 * I * H * 2
+    w2_bytes = E * H * I * 2
+    # algorithmic bytes of one GEMM1 launch: W1 once + the B token rows once + the SwiGLU output
+    gemm1_bytes = w1_bytes + B * H * 2 + B * k * I * 2
+    gemm1_ms = kern["gemm1_gather_swiglu"][1]
+    res = {
+        "ms_per_step": ms,
+        "tokens_per_s": B / ms * 1e3,
+        "tflops": flops / ms / 1e9,
+        "weight_gbs": (w1_bytes + w2_bytes) / ms / 1e6,
+        "kernels_us": {name: round(v[1] * 1e3, 2) for name, v in kern.items()},
+        "gemm1_ms": gemm1_ms,
+        "gemm1_bytes": gemm1_bytes,
+        "gemm1_flops": 2.0 * B * k * H * 2 * I,
+    }
+    return res, (raw[0], t, layers[0], out)
+
+
+def cpu_baseline_moe(torch, state, n_tok):
+    """The oracle's restatement of run.cpp:625-704 on the first n_tok tokens, all host threads."""
+    from oracle import oracle as orc
+    raw, t, layer, _ = state
+    f = lambda x: x.float().cpu().numpy()
+    args = [f(raw[nm]) for nm in ("w_router", "b_router", "w1", "b1", "w2", "b2")]
+    tt = f(t[:n_tok])
+    t0 = time.perf_counter()
+    want = orc.moe_layer(tt, *args, k=4, limit=7.0, stage=orc.STAGE_SWIGLU)
+    dt = time.perf_counter() - t0
+    # the timed sample doubles as a parity check of the benchmarked tensors
+    got = layer.forward(t[:n_tok].contiguous()).cpu().numpy()
+    import numpy as np
+    d = np.abs(got - want)
+    rel_max = float(d.max() / np.abs(want).max())
+    rel_mean = float(d.mean() / np.abs(want).mean())
+    return {"value": n_tok / dt, "unit": "tokens/s", "cores": orc.num_threads(), "kind": "port",
+            "sample": f"first {n_tok} of the {t.shape[0]} tokens, same tensors, {dt:.1f} s",
+            "parity_vs_gpu": {"max_rel": rel_max, "mean_rel": rel_mean}}
+
+
+def bench_attn(ops, torch, steps, warmup):
+    import numpy as np
+    B, n_q, n_kv, D, S = 256, 64, 8, 64, 4096
+    rng = np.random.default_rng(0)
+    lens_np = rng.integers(512, 4097, size=B).astype(np.int32)
+    lens = torch.from_numpy(lens_np).cuda()
+    caches = []
+    for _ in range(2):
+        c = ops.KVCache(B, n_kv, D, S)
+        c.k.normal_()
+        c.v.normal_()
+        caches.append(c)
+    q = torch.randn(B, n_q, D, device="cuda")
+    sinks = torch.randn(n_q, device="cuda")
+    attn = ops.AttnDecode(B, n_q, n_kv, D, S)
+    out = torch.empty(B, n_q, D, dtype=torch.bfloat16, device="cuda")
+    res = {}
+    for name, window in (("full", 0), ("window128", 128)):
+        for i in range(warmup):
+            attn.forward(q, caches[i % 2], lens, sinks, window=window, out=out)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(steps):
+            attn.forward(q, caches[i % 2], lens, sinks, window=window, out=out)
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) * 1e3 / steps
+        act = np.minimum(lens_np, window) if window else lens_np
+        kv_bytes = int(act.sum()) * n_kv * D * 2 * 2
+        res[name] = {"us": round(ms * 1e3, 1), "kv_mb": round(kv_bytes / 1e6, 1),
+                     "gbs": round(kv_bytes / ms / 1e6, 1),
+                     "hbm_frac": round(kv_bytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
+    return res
+
+
+def main():
+    args = parse()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.stderr.write("bench.py: this build runs on ONE GPU (all experts on one MI355X); "
+                         "--gpus N with N > 1 is not supported\n")
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        sys.stderr.write("bench.py: no GPU visible; there is no CPU path to benchmark\n")
+        sys.exit(3)
+    importlib.import_module("gpt-oss-team01_amd.lib").load()
+    ops = importlib.import_module("gpt-oss-team01_amd.ops")
+
+    # a plain device copy of known size (2 x 1 GiB moved), so counter runs of this same command can
+    # be scaled by what the counters read for it
+    src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda")
+    dst = torch.empty_like(src)
+    for _ in range(3):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    del src, dst
+    torch.cuda.empty_cache()
+
+    moe, state = bench_moe(ops, torch, args)
+    cpu = cpu_baseline_moe(torch, state, args.cpu_tokens) if args.cpu_tokens > 0 else None
+    del state
+    torch.cuda.empty_cache()
+    extra = {"moe_tflops": round(moe["tflops"], 1),
+             "moe_mfma_frac": round(moe["tflops"] / MFMA_BF16_PEAK_TFLOPS, 4),
+             "moe_weight_gbs": round(moe["weight_gbs"], 1),
+             "moe_weight_hbm_frac": round(moe["weight_gbs"] / HBM_PEAK_GBS, 4),
+             "moe_kernels_us": moe["kernels_us"],
+             "gemm1_tflops": round(moe["gemm1_flops"] / moe["gemm1_ms"] / 1e9, 1)}
+    if not args.no_attn:
+        extra["decode_attn"] = bench_attn(ops, torch, max(10, args.steps // 2), args.warmup)
+
+    achieved = moe["gemm1_bytes"] / moe["gemm1_ms"] / 1e6
+    line = {
+        "metric": "MoE-layer tokens/s (GPT-OSS-20B layer shape, 1024 tokens, 1 GPU)",
+        "value": round(moe["tokens_per_s"], 1),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(moe["ms_per_step"], 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "configs[1]: single GPT-OSS-20B MoE layer, isolated",
+                   "tokens": args.tokens, "hidden": 2880, "experts": 32, "top_k": 4,
+                   "intermediate": 2880, "weights": "bf16 N(0,0.02), two sets alternated",
+                   "activations": "bf16 N(0,1)"},
+        "roofline": {"kernel": "grouped_gemm_kernel<8,true,1> (gather + GEMM1 + SwiGLU)",
+                     "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "bytes_per_launch": moe["gemm1_bytes"],
+                     "avg_launch_us": round(moe["gemm1_ms"] * 1e3, 2)},
+        "cpu_baseline": cpu,
+        "extra": extra,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

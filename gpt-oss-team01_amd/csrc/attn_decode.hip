@@ -409,12 +409,16 @@ extern "C" int gptoss_attn_decode(const float *q, const void *k_cache, const voi
   hipStream_t s = (hipStream_t)stream;
   long long items = (long long)B * n_kv * pl.max_chunks;
   int grid = (int)((items + 3) / 4);
-  if (head_dim == 64) attn_decode_kernel<64><<<grid, 256, 0, s>>>(p);
-  else attn_decode_kernel<32><<<grid, 256, 0, s>>>(p);
+  {
+    TraceScope ts("attn_decode", s);
+    if (head_dim == 64) attn_decode_kernel<64><<<grid, 256, 0, s>>>(p);
+    else attn_decode_kernel<32><<<grid, 256, 0, s>>>(p);
+  }
   GPTOSS_LAUNCH_CHECK("attn_decode_kernel");
   if (pl.max_chunks > 1) {
     int per_block = 256 / head_dim;
     int rgrid = (B * n_q + per_block - 1) / per_block;
+    TraceScope ts("attn_reduce", s);
     if (head_dim == 64) attn_reduce_kernel<64><<<rgrid, 256, 0, s>>>(p);
     else attn_reduce_kernel<32><<<rgrid, 256, 0, s>>>(p);
     GPTOSS_LAUNCH_CHECK("attn_reduce_kernel");

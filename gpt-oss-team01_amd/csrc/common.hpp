@@ -33,6 +33,16 @@ int fail(int code, const char *fmt, ...);
       return ::gptoss::fail(GPTOSS_ERR_HIP, "launch %s: %s", name, hipGetErrorString(err__)); \
   } while (0)
 
+// ---- kernel timing hook (host) ----------------------------------------------------------------
+// When the calling thread has armed a trace (gptoss_trace_set), every kernel launch made by an
+// entry point is bracketed by a start/stop event pair on the launch stream.
+struct TraceScope {
+  TraceScope(const char *name, hipStream_t stream);
+  ~TraceScope();
+  int slot;
+  hipStream_t stream;
+};
+
 static inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 static inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 static inline int cdiv(int a, int b) { return (a + b - 1) / b; }

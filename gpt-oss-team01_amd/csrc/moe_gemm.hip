@@ -329,7 +329,10 @@ static int launch_gemm(const GemmParams &p, int max_tiles, hipStream_t s) {
   int total = max_tiles * p.n_col_tiles;
   int grid = ((total + 7) / 8) * 8;
   if (grid == 0) return GPTOSS_OK;
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(GEMM_THREADS), smem, s, p);
+  {
+    TraceScope ts(GATHER ? "gemm1_gather_swiglu" : (EPI == EPI_F32 ? "gemm_f32" : (EPI == EPI_BF16 ? "gemm_bf16" : "gemm_swiglu")), s);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(GEMM_THREADS), smem, s, p);
+  }
   GPTOSS_LAUNCH_CHECK("grouped_gemm_kernel");
   return GPTOSS_OK;
 }
@@ -356,7 +359,10 @@ int run_gemm(const GemmParams &p, bool gather, int epi, int rows_per_tile, int m
 int run_combine(const float *y2, const float *topk_w, const int *inv_perm, float *out, int B, int H,
                 int k, int accumulate, hipStream_t s) {
   if (B == 0) return GPTOSS_OK;
-  combine_kernel<<<B, 256, 0, s>>>(y2, topk_w, inv_perm, out, H, k, accumulate);
+  {
+    TraceScope ts("combine", s);
+    combine_kernel<<<B, 256, 0, s>>>(y2, topk_w, inv_perm, out, H, k, accumulate);
+  }
   GPTOSS_LAUNCH_CHECK("combine_kernel");
   return GPTOSS_OK;
 }

@@ -247,6 +247,7 @@ extern "C" int gptoss_router_gemm(const void *t, const void *w_router, const flo
   dim3 grid(cdiv(B, 16)), block(256);
   const bf16_t *tp = (const bf16_t *)t, *wp = (const bf16_t *)w_router;
   int nb = cdiv(E, 16);
+  TraceScope ts("router_gemm", s);
   if (nb <= 1) router_gemm_kernel<1><<<grid, block, 0, s>>>(tp, wp, b_router, logits, B, H, E);
   else if (nb <= 2) router_gemm_kernel<2><<<grid, block, 0, s>>>(tp, wp, b_router, logits, B, H, E);
   else if (nb <= 4) router_gemm_kernel<4><<<grid, block, 0, s>>>(tp, wp, b_router, logits, B, H, E);
@@ -279,6 +280,7 @@ extern "C" int gptoss_moe_route(const float *logits, int B, int E, int k, float 
   if (B > 0) {
     dim3 grid(cdiv(B * 32, 256)), block(256);
     int nj = cdiv(E, 32);
+    TraceScope ts("topk_softmax", s);
     if (nj <= 1) topk_softmax_kernel<1><<<grid, block, 0, s>>>(logits, B, E, k, topk_w, topk_i);
     else if (nj <= 2) topk_softmax_kernel<2><<<grid, block, 0, s>>>(logits, B, E, k, topk_w, topk_i);
     else if (nj <= 4) topk_softmax_kernel<4><<<grid, block, 0, s>>>(logits, B, E, k, topk_w, topk_i);
@@ -288,9 +290,12 @@ extern "C" int gptoss_moe_route(const float *logits, int B, int E, int k, float 
   int nbits = 0;
   while ((1 << nbits) < E) nbits++;
   size_t smem = sizeof(int) * ((size_t)SORT_WAVES * E + E + (E + 1));
-  group_sort_kernel<<<1, SORT_THREADS, smem, s>>>(topk_i, B * k, E, nbits, expert_offsets,
-                                                  sorted_pair_ids, inv_perm,
-                                                  rows_per_tile ? tiles : nullptr, rows_per_tile);
+  {
+    TraceScope ts("group_sort", s);
+    group_sort_kernel<<<1, SORT_THREADS, smem, s>>>(topk_i, B * k, E, nbits, expert_offsets,
+                                                    sorted_pair_ids, inv_perm,
+                                                    rows_per_tile ? tiles : nullptr, rows_per_tile);
+  }
   GPTOSS_LAUNCH_CHECK("group_sort_kernel");
   return GPTOSS_OK;
 }

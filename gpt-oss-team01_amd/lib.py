@@ -53,6 +53,9 @@ _vp, _i, _sz, _f = C.c_void_p, C.c_int, C.c_size_t, C.c_float
 SIGNATURES = {
     "gptoss_last_error_string": (C.c_char_p, []),
     "gptoss_abi_version": (_i, []),
+    "gptoss_trace_set": (_i, [_vp, _vp, _i]),
+    "gptoss_trace_count": (_i, []),
+    "gptoss_trace_name": (C.c_char_p, [_i]),
     "gptoss_packed_weight_bytes": (_sz, [_i, _i, _i]),
     "gptoss_pack_weight": (_i, [_vp, _vp, _i, _i, _i, _i, _vp]),
     "gptoss_router_gemm": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]),

@@ -176,3 +176,47 @@ class AttnDecode:
                                            cache.cap, window, max_len or self.max_len,
                                            _ptr(self.ws), self.ws_bytes, _stream()))
         return out
+
+
+class KernelTrace:
+    """Per-kernel HIP-event timing of the entry points called inside the ``with`` block
+    (events are recorded on the stream each kernel is launched on)."""
+
+    def __init__(self, capacity=4096):
+        _need_gpu()
+        self.L = _l.load()
+        self.capacity = capacity
+        self._start = [torch.cuda.Event(enable_timing=True) for _ in range(capacity)]
+        self._stop = [torch.cuda.Event(enable_timing=True) for _ in range(capacity)]
+        # torch creates the underlying hipEvent_t lazily, at the first record()
+        for e in self._start + self._stop:
+            e.record()
+        torch.cuda.synchronize()
+        self._sa = (C.c_void_p * capacity)(*[e.cuda_event for e in self._start])
+        self._so = (C.c_void_p * capacity)(*[e.cuda_event for e in self._stop])
+        self.count = 0
+
+    def __enter__(self):
+        _l.check(self.L.gptoss_trace_set(self._sa, self._so, self.capacity))
+        return self
+
+    def __exit__(self, *exc):
+        # labels are read before the trace is disarmed
+        self.count = self.L.gptoss_trace_count()
+        self._names = [self.L.gptoss_trace_name(i).decode() for i in range(self.count)]
+        self.L.gptoss_trace_set(None, None, 0)
+        return False
+
+    def results(self):
+        """-> list of (kernel label, milliseconds), in launch order.  Synchronises."""
+        torch.cuda.synchronize()
+        return [(self._names[i], self._start[i].elapsed_time(self._stop[i]))
+                for i in range(self.count)]
+
+    def summary(self):
+        """-> {label: (calls, mean ms)}"""
+        agg = {}
+        for name, ms in self.results():
+            c, t = agg.get(name, (0, 0.0))
+            agg[name] = (c + 1, t + ms)
+        return {k: (c, t / c) for k, (c, t) in agg.items()}

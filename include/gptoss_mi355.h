@@ -47,6 +47,16 @@ const char *gptoss_last_error_string(void);
 /* ABI version of this header (major*100+minor). */
 int gptoss_abi_version(void);
 
+/* Kernel timing hook.  Replaces the reference's GpuTimer (getp-csrc/include/utils.hpp:13-39, a
+ * hipEvent pair around each op, compiled in with -DTIME_GPU).  After gptoss_trace_set(start, stop,
+ * n) with two arrays of n hipEvent_t created by the caller, every kernel launched by an entry point
+ * called from this thread records start[i] / stop[i] around itself on its stream (i counts
+ * launches since the call).  gptoss_trace_set(NULL, NULL, 0) disarms.  gptoss_trace_name(i) is the
+ * label of launch i.  The caller synchronises before reading the events. */
+int gptoss_trace_set(void *const *start_events, void *const *stop_events, int n);
+int gptoss_trace_count(void);
+const char *gptoss_trace_name(int i);
+
 /* ------------------------------------------------------------------ weight layout ---------- */
 
 /* Flags for gptoss_pack_weight. */
