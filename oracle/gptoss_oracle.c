@@ -392,6 +392,7 @@ typedef struct {
   float *key_cache, *value_cache; /* [L, seq_len, kv_dim] */
   float *cos_t, *sin_t;           /* [seq_len, D/2] */
   int stage;
+  float min_router_gap; /* smallest (k-th - (k+1)-th) router score seen by orc_forward */
 } OrcModel;
 
 long long orc_weight_floats(const OrcConfig *c) {
@@ -407,6 +408,7 @@ OrcModel *orc_model_create(const OrcConfig *cfg, const float *weights, int stage
   OrcModel *m = (OrcModel *)calloc(1, sizeof(OrcModel));
   m->cfg = *cfg;
   m->stage = stage;
+  m->min_router_gap = INFINITY;
   const OrcConfig *c = cfg;
   long long H = c->hidden_dim, V = c->vocab_size, L = c->n_layers, E = c->n_experts;
   long long D = c->head_dim, nq = c->n_attn_heads, nkv = c->n_kv_heads, I = c->intermediate_dim;
@@ -460,6 +462,7 @@ void orc_model_destroy(OrcModel *m) {
 
 float *orc_model_logits(OrcModel *m) { return m->logits; }
 float *orc_model_x(OrcModel *m) { return m->x; }
+float orc_model_min_router_gap(OrcModel *m) { return m->min_router_gap; }
 
 static void round_vec(float *x, long long n) {
   for (long long i = 0; i < n; i++) x[i] = bf16_round(x[i]);
@@ -558,6 +561,15 @@ float *orc_forward(OrcModel *m, int token, int pos) {
     mm(m, m->score, m->t, m->w_router + l * hidden_dim * E, hidden_dim, E);
     for (int i = 0; i < E; i++) m->score[i] += m->b_router[l * E + i];
     orc_topk_softmax(m->score, 1, E, k, m->topk_v, m->topk_i);
+    if (k < E) {
+      float kth = m->score[m->topk_i[k - 1]], next = -INFINITY;
+      for (int i = 0; i < E; i++) {
+        int picked = 0;
+        for (int j = 0; j < k; j++) picked |= (m->topk_i[j] == i);
+        if (!picked && m->score[i] > next) next = m->score[i];
+      }
+      if (kth - next < m->min_router_gap) m->min_router_gap = kth - next;
+    }
     memset(m->e_agg, 0, hidden_dim * sizeof(float));
     for (int e = 0; e < E; e++) {
       float expert_w = 0;
@@ -614,12 +626,14 @@ int orc_argmax(const float *v, int n) {
  *   prompts [n_req, prompt_stride] with n_prompt[r] valid ids each
  *   out     [n_req, max_seq_len+1]
  *   margins (optional) [n_req, max_seq_len+1]: top1-top2 logit gap of every sampled position
+ *   min_router_gap (optional): smallest gap between the k-th and (k+1)-th router score met
  * Returns the number of generated tokens counted the way the harness counts them.
  */
 long long orc_generate(const OrcConfig *cfg, const float *weights, int stage, const int *prompts,
                        const int *n_prompt, int prompt_stride, int n_req, int max_seq_len,
-                       int *out, float *margins) {
+                       int *out, float *margins, float *min_router_gap) {
   long long total = 0;
+  if (min_router_gap) *min_router_gap = INFINITY;
   for (int r = 0; r < n_req; r++) {
     OrcModel *m = orc_model_create(cfg, weights, stage);
     const int *pt = prompts + 1ll * r * prompt_stride;
@@ -649,6 +663,7 @@ long long orc_generate(const OrcConfig *cfg, const float *weights, int stage, co
     if (generated_len < 0) generated_len = 0;
     o[generated_len + 1] = -1;
     total += generated_len + 1;
+    if (min_router_gap && m->min_router_gap < *min_router_gap) *min_router_gap = m->min_router_gap;
     orc_model_destroy(m);
   }
   return total;

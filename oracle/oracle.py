@@ -237,9 +237,11 @@ def generate(cfg, weights_flat, prompts, max_seq_len, stage=0, want_margins=Fals
     oc = OrcConfig.from_config(cfg)
     out = np.zeros((n_req, max_seq_len + 1), np.int32)
     margins = np.zeros((n_req, max_seq_len + 1), np.float32)
+    gap = C.c_float(0)
     n = lib().orc_generate(C.byref(oc), _fp(w), C.c_int(stage), _ip(prompts), _ip(n_prompt),
                            C.c_int(stride), C.c_int(n_req), C.c_int(max_seq_len), _ip(out),
-                           _fp(margins))
+                           _fp(margins), C.byref(gap))
+    generate.last_min_router_gap = float(gap.value)
     if want_margins:
         return out, int(n), margins
     return out, int(n)
