@@ -374,7 +374,7 @@ extern "C" int gptoss_attn_decode(const float *q, const void *k_cache, const voi
                  "attn_decode: head_dim must be 32 or 64 (got %d)", head_dim);
   GPTOSS_REQUIRE(capacity > 0 && capacity % 64 == 0 && window >= 0 && max_len > 0, GPTOSS_ERR_DIM,
                  "attn_decode: need capacity %% 64 == 0, window >= 0, max_len > 0 (capacity=%d)", capacity);
-  GPTOSS_REQUIRE(window == 0 ? max_len <= capacity : window <= capacity, GPTOSS_ERR_DIM,
+  GPTOSS_REQUIRE(max_len <= capacity || (window > 0 && window <= capacity), GPTOSS_ERR_DIM,
                  "attn_decode: the cache must hold every active position (capacity=%d window=%d max_len=%d)",
                  capacity, window, max_len);
   GPTOSS_REQUIRE(aligned(q, 16) && aligned(k_cache, 16) && aligned(v_cache, 16) && aligned(out, 8),

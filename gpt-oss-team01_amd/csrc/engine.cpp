@@ -1,0 +1,495 @@
+// Single-GPU decode engine: device weights in kernel layout, run state, one lock-step decode step
+// (the op order of the reference's forward_gpu_20b_batched, getp-csrc/src/model.cpp:6-151) and the
+// greedy generation loop of its getp scheduler (getp-csrc/submit/getp_run_submit.cpp:60-96).
+#include <math.h>
+#include <string.h>
+
+#include <algorithm>
+#include <vector>
+
+#include "common.hpp"
+#include "gemm.hpp"
+#include "glue.hpp"
+
+#ifndef M_PI
+#define M_PI 3.14159265358979323846
+#endif
+
+namespace gptoss {
+
+struct LayerWeights {
+  float *attn_norm, *mlp_norm;    // fp32 [H]
+  bf16_t *w_qkv;                  // packed [(nq+2nkv)D, H]
+  float *b_qkv;
+  bf16_t *w_o;                    // packed [H, nq*D]
+  float *b_o;
+  float *sinks;                   // [nq]
+  bf16_t *w_router;               // [E,H] row-major
+  float *b_router;
+  bf16_t *w1;                     // packed GLU [E][2I,H]
+  float *b1;
+  bf16_t *w2;                     // packed [E][H,I]
+  float *b2;
+  bf16_t *k_cache, *v_cache;
+  int cache_cap;
+  int window;                     // 0 = full attention
+};
+
+}  // namespace gptoss
+
+using namespace gptoss;
+
+struct gptoss_engine {
+  gptoss_config cfg;
+  int max_batch, max_seq, flags;
+  hipStream_t stream;
+  std::vector<void *> allocs;
+  // weights
+  bf16_t *embedding;   // [V,H]
+  bf16_t *unembedding; // packed [V,H]
+  float *final_norm;
+  std::vector<LayerWeights> layers;
+  float *cos_t, *sin_t;  // [max_seq, D/2]
+  // run state
+  int *d_tokens, *d_next, *d_lens;
+  int *h_tokens, *h_next;  // pinned
+  float *x, *qkv, *q, *tb2, *logits;
+  bf16_t *t, *attn_out;
+  void *moe_ws, *attn_ws;
+  size_t moe_ws_bytes, attn_ws_bytes;
+  size_t device_bytes;
+};
+
+namespace {
+
+struct Builder {
+  gptoss_engine *e;
+  int rc = GPTOSS_OK;
+  // staging for the fp32 -> device layout conversion
+  float *stage_f32 = nullptr;
+  bf16_t *stage_bf16 = nullptr;
+  size_t stage_elems = 0;
+
+  template <typename T>
+  T *alloc(size_t n) {
+    if (rc != GPTOSS_OK) return nullptr;
+    void *p = nullptr;
+    size_t bytes = align_up(n * sizeof(T), 256);
+    hipError_t err = hipMalloc(&p, bytes);
+    if (err != hipSuccess) {
+      rc = fail(GPTOSS_ERR_HIP, "engine: hipMalloc of %zu bytes failed: %s", bytes, hipGetErrorString(err));
+      return nullptr;
+    }
+    e->allocs.push_back(p);
+    e->device_bytes += bytes;
+    return (T *)p;
+  }
+
+  bool ok() const { return rc == GPTOSS_OK; }
+  void check(int r) { if (rc == GPTOSS_OK && r != GPTOSS_OK) rc = r; }
+  void hip(hipError_t err, const char *what) {
+    if (rc == GPTOSS_OK && err != hipSuccess) rc = fail(GPTOSS_ERR_HIP, "engine: %s: %s", what, hipGetErrorString(err));
+  }
+
+  // fp32 host tensor -> fp32 device tensor
+  float *upload_f32(const float *host, size_t n, uint64_t seed, float mean, float std) {
+    float *d = alloc<float>(n);
+    if (!ok()) return nullptr;
+    if (host) hip(hipMemcpyAsync(d, host, n * sizeof(float), hipMemcpyHostToDevice, e->stream), "H2D");
+    else check(run_synth_f32(d, n, seed, mean, std, e->stream));
+    return d;
+  }
+
+  // fp32 host matrices -> bf16 device matrices, row-major (pack == false) or fragment order
+  bf16_t *upload_matrices(const float *host, int n_mat, int n_out, int n_in, bool pack, int pack_flags,
+                          uint64_t seed, float std) {
+    size_t per = (size_t)n_out * n_in;
+    bf16_t *dst = alloc<bf16_t>(per * n_mat);
+    if (!ok()) return nullptr;
+    int group = (int)std::max<size_t>(1, stage_elems / per);
+    if (per > stage_elems) {
+      rc = fail(GPTOSS_ERR_DIM, "engine: a %d x %d matrix exceeds the staging buffer", n_out, n_in);
+      return nullptr;
+    }
+    for (int m0 = 0; m0 < n_mat && ok(); m0 += group) {
+      int nm = std::min(group, n_mat - m0);
+      size_t n = per * nm;
+      const void *src;
+      int flags = pack_flags;
+      if (host) {
+        hip(hipMemcpyAsync(stage_f32, host + per * m0, n * sizeof(float), hipMemcpyHostToDevice, e->stream), "H2D");
+        src = stage_f32;
+        flags |= GPTOSS_PACK_SRC_FP32;
+      } else {
+        check(run_synth_bf16(stage_bf16, n, seed + 7919ull * (uint64_t)m0, 0.f, std, e->stream));
+        src = stage_bf16;
+      }
+      if (!ok()) break;
+      if (pack) {
+        check(gptoss_pack_weight(src, dst + per * m0, nm, n_out, n_in, flags, e->stream));
+      } else if (host) {
+        check(run_f32_to_bf16(stage_f32, dst + per * m0, n, e->stream));
+      } else {
+        hip(hipMemcpyAsync(dst + per * m0, stage_bf16, n * sizeof(bf16_t), hipMemcpyDeviceToDevice, e->stream), "D2D");
+      }
+      // the staging buffer is reused by the next group
+      hip(hipStreamSynchronize(e->stream), "sync");
+    }
+    return dst;
+  }
+};
+
+// cos/sin tables with the float arithmetic of run.cpp:404-478 (ntk_beta 32, ntk_alpha 1)
+void rope_tables(const gptoss_config &c, int n_pos, std::vector<float> &cs, std::vector<float> &sn) {
+  const int d_half = c.head_dim / 2;
+  std::vector<float> inv_freq(d_half);
+  const float base = c.rope_theta, scaling_factor = c.rope_scaling_factor;
+  const float initial_context_length = (float)c.initial_context_length;
+  const float ntk_beta = 32.0f, ntk_alpha = 1.0f;
+  float concentration;
+  std::vector<float> freq(d_half);
+  for (int i = 0; i < d_half; i++) freq[i] = powf(base, ((float)(2 * i)) / (float)c.head_dim);
+  if (scaling_factor > 1.0f) {
+    concentration = 0.1f * logf(scaling_factor) + 1.0f;
+    float low = d_half * logf(initial_context_length / (ntk_beta * 2.0f * M_PI)) / logf(base);
+    float high = d_half * logf(initial_context_length / (ntk_alpha * 2.0f * M_PI)) / logf(base);
+    for (int i = 0; i < d_half; i++) {
+      float interpolation = 1.0f / (scaling_factor * freq[i]);
+      float extrapolation = 1.0f / freq[i];
+      float ramp = ((float)i - low) / (high - low);
+      if (ramp < 0) ramp = 0;
+      if (ramp > 1) ramp = 1;
+      float mask = 1.0f - ramp;
+      inv_freq[i] = interpolation * (1.0f - mask) + extrapolation * mask;
+    }
+  } else {
+    concentration = 1.0f;
+    for (int i = 0; i < d_half; i++) inv_freq[i] = 1.0f / freq[i];
+  }
+  cs.resize((size_t)n_pos * d_half);
+  sn.resize((size_t)n_pos * d_half);
+  for (int pos = 0; pos < n_pos; pos++)
+    for (int j = 0; j < d_half; j++) {
+      float val = (float)pos * inv_freq[j];
+      cs[(size_t)pos * d_half + j] = cosf(val) * concentration;
+      sn[(size_t)pos * d_half + j] = sinf(val) * concentration;
+    }
+}
+
+int dense_gemm(const bf16_t *A, const bf16_t *W, const float *bias, void *out, int epi, int B, int N,
+               int K, hipStream_t s) {
+  GemmParams g{};
+  g.A = A;
+  g.W = W;
+  g.bias = bias;
+  g.out = out;
+  g.tiles = nullptr;
+  g.dense_rows = B;
+  g.N = N;
+  g.K = K;
+  g.n_col_tiles = cdiv(N, 256);
+  int rpt = B > 128 ? 256 : (B > 64 ? 128 : (B > 32 ? 64 : 32));
+  return run_gemm(g, false, epi, rpt, cdiv(B, rpt), s);
+}
+
+void destroy(gptoss_engine *e) {
+  if (!e) return;
+  for (void *p : e->allocs) (void)hipFree(p);
+  if (e->h_tokens) (void)hipHostFree(e->h_tokens);
+  if (e->h_next) (void)hipHostFree(e->h_next);
+  if (e->stream) (void)hipStreamDestroy(e->stream);
+  delete e;
+}
+
+}  // namespace
+
+extern "C" int gptoss_engine_create(const gptoss_config *cfg, const float *host_weights, int max_batch,
+                                    int max_seq, int flags, uint64_t seed, gptoss_engine **out) {
+  GPTOSS_REQUIRE(cfg && out, GPTOSS_ERR_NULL, "engine_create: null pointer");
+  *out = nullptr;
+  const bool synthetic = (flags & GPTOSS_ENGINE_SYNTHETIC) != 0;
+  GPTOSS_REQUIRE(synthetic || host_weights, GPTOSS_ERR_NULL, "engine_create: host_weights is NULL");
+  GPTOSS_REQUIRE(!(flags & GPTOSS_ENGINE_PRECISE), GPTOSS_ERR_STATE,
+                 "engine_create: GPTOSS_ENGINE_PRECISE is not available in this build");
+  const gptoss_config &c = *cfg;
+  const int H = c.hidden_dim, V = c.vocab_size, L = c.n_layers, E = c.n_experts, k = c.experts_per_token;
+  const int D = c.head_dim, nq = c.n_attn_heads, nkv = c.n_kv_heads, I = c.intermediate_dim;
+  GPTOSS_REQUIRE(H > 0 && V > 0 && L > 0 && E > 0 && k > 0 && D > 0 && nq > 0 && nkv > 0 && I > 0,
+                 GPTOSS_ERR_DIM, "engine_create: non-positive model dimension");
+  const int qkv_dim = (nq + 2 * nkv) * D;
+  GPTOSS_REQUIRE(H % 64 == 0 && I % 64 == 0 && qkv_dim % 64 == 0 && (nq * D) % 64 == 0 && V % 64 == 0,
+                 GPTOSS_ERR_DIM,
+                 "engine_create: hidden, intermediate, (n_q+2n_kv)*head_dim, n_q*head_dim and vocab must be "
+                 "multiples of 64 (H=%d I=%d qkv=%d V=%d)", H, I, qkv_dim, V);
+  GPTOSS_REQUIRE((D == 32 || D == 64) && nq % nkv == 0 && nq / nkv <= 16, GPTOSS_ERR_DIM,
+                 "engine_create: head_dim must be 32 or 64 and n_q/n_kv <= 16");
+  GPTOSS_REQUIRE(E <= 256 && k <= 8 && k <= E, GPTOSS_ERR_DIM, "engine_create: need E <= 256, k <= min(8,E)");
+  GPTOSS_REQUIRE(max_batch >= 1 && max_seq >= 1 && max_seq <= c.seq_len, GPTOSS_ERR_DIM,
+                 "engine_create: need max_batch >= 1 and 1 <= max_seq <= seq_len (%d)", c.seq_len);
+  GPTOSS_REQUIRE(c.sliding_window >= 0, GPTOSS_ERR_DIM, "engine_create: negative sliding window");
+
+  gptoss_engine *e = new gptoss_engine();
+  e->cfg = c;
+  e->max_batch = max_batch;
+  e->max_seq = max_seq;
+  e->flags = flags;
+  e->device_bytes = 0;
+  e->h_tokens = e->h_next = nullptr;
+  e->stream = nullptr;
+  Builder b;
+  b.e = e;
+  b.hip(hipStreamCreate(&e->stream), "hipStreamCreate");
+  b.hip(hipHostMalloc((void **)&e->h_tokens, sizeof(int) * max_batch, hipHostMallocDefault), "hipHostMalloc");
+  b.hip(hipHostMalloc((void **)&e->h_next, sizeof(int) * max_batch, hipHostMallocDefault), "hipHostMalloc");
+
+  // staging: large enough for one expert's gate/up matrix, one qkv matrix and a slice of the
+  // (un)embedding table
+  size_t biggest = std::max({(size_t)2 * I * H, (size_t)qkv_dim * H, (size_t)H * nq * D, (size_t)E * H});
+  b.stage_elems = std::max<size_t>(biggest, (size_t)16 << 20);
+  if (!synthetic) b.hip(hipMalloc((void **)&b.stage_f32, b.stage_elems * sizeof(float)), "staging hipMalloc");
+  else b.hip(hipMalloc((void **)&b.stage_bf16, b.stage_elems * sizeof(bf16_t)), "staging hipMalloc");
+
+  // walk the .bin payload in file order (reference run.cpp:194-233)
+  const float *p = host_weights;
+  auto take = [&](size_t n) -> const float * {
+    if (synthetic) return nullptr;
+    const float *r = p;
+    p += n;
+    return r;
+  };
+  uint64_t sd = seed * 1000003ull + 17;
+  auto next_seed = [&]() { return sd += 0x9E3779B97F4A7C15ull; };
+  const float STD = 0.02f;
+
+  // embedding rows are gathered, not multiplied: row-major bf16.  Upload in row slices.
+  {
+    const float *emb = take((size_t)V * H);
+    const float *unemb = take((size_t)V * H);
+    int rows_per = (int)std::max<size_t>(64, (b.stage_elems / H) / 64 * 64);
+    e->embedding = b.alloc<bf16_t>((size_t)V * H);
+    e->unembedding = b.alloc<bf16_t>((size_t)V * H);
+    for (int pass = 0; pass < 2 && b.ok(); pass++) {
+      const float *src = pass == 0 ? emb : unemb;
+      bf16_t *dst = pass == 0 ? e->embedding : e->unembedding;
+      for (int r0 = 0; r0 < V && b.ok(); r0 += rows_per) {
+        int nr = std::min(rows_per, V - r0);
+        size_t n = (size_t)nr * H;
+        const void *s;
+        int fl = 0;
+        if (src) {
+          b.hip(hipMemcpyAsync(b.stage_f32, src + (size_t)r0 * H, n * sizeof(float), hipMemcpyHostToDevice, e->stream), "H2D");
+          s = b.stage_f32;
+          fl = GPTOSS_PACK_SRC_FP32;
+        } else {
+          b.check(run_synth_bf16(b.stage_bf16, n, next_seed(), 0.f, STD, e->stream));
+          s = b.stage_bf16;
+        }
+        if (!b.ok()) break;
+        if (pass == 0) {
+          if (src) b.check(run_f32_to_bf16(b.stage_f32, dst + (size_t)r0 * H, n, e->stream));
+          else b.hip(hipMemcpyAsync(dst + (size_t)r0 * H, b.stage_bf16, n * sizeof(bf16_t), hipMemcpyDeviceToDevice, e->stream), "D2D");
+        } else {
+          // fragment order is blocked by 32 output rows, so a slice of rows packs independently
+          b.check(gptoss_pack_weight(s, dst + (size_t)r0 * H, 1, nr, H, fl, e->stream));
+        }
+        b.hip(hipStreamSynchronize(e->stream), "sync");
+      }
+    }
+  }
+  const float *attn_norm = take((size_t)L * H), *mlp_norm = take((size_t)L * H), *fin = take(H);
+  const float *w_qkv = take((size_t)L * qkv_dim * H), *b_qkv = take((size_t)L * qkv_dim);
+  const float *w_o = take((size_t)L * H * nq * D), *b_o = take((size_t)L * H);
+  const float *sinks = take((size_t)L * nq);
+  const float *w_router = take((size_t)L * E * H), *b_router = take((size_t)L * E);
+  const float *w1 = take((size_t)L * E * 2 * I * H), *b1 = take((size_t)L * E * 2 * I);
+  const float *w2 = take((size_t)L * E * H * I), *b2 = take((size_t)L * E * H);
+  auto at = [&](const float *base, size_t per, int l) -> const float * { return base ? base + per * l : nullptr; };
+
+  e->final_norm = b.upload_f32(fin, H, next_seed(), 1.f, STD);
+  e->layers.resize(L);
+  const int W = c.sliding_window;
+  const int cap_full = (int)align_up((size_t)max_seq, 64);
+  for (int l = 0; l < L && b.ok(); l++) {
+    LayerWeights &w = e->layers[l];
+    w.attn_norm = b.upload_f32(at(attn_norm, H, l), H, next_seed(), 1.f, STD);
+    w.mlp_norm = b.upload_f32(at(mlp_norm, H, l), H, next_seed(), 1.f, STD);
+    w.w_qkv = b.upload_matrices(at(w_qkv, (size_t)qkv_dim * H, l), 1, qkv_dim, H, true, 0, next_seed(), STD);
+    w.b_qkv = b.upload_f32(at(b_qkv, qkv_dim, l), qkv_dim, next_seed(), 0.f, STD);
+    w.w_o = b.upload_matrices(at(w_o, (size_t)H * nq * D, l), 1, H, nq * D, true, 0, next_seed(), STD);
+    w.b_o = b.upload_f32(at(b_o, H, l), H, next_seed(), 0.f, STD);
+    w.sinks = b.upload_f32(at(sinks, nq, l), nq, next_seed(), 0.f, STD);
+    w.w_router = b.upload_matrices(at(w_router, (size_t)E * H, l), 1, E, H, false, 0, next_seed(), STD);
+    w.b_router = b.upload_f32(at(b_router, E, l), E, next_seed(), 0.f, STD);
+    w.w1 = b.upload_matrices(at(w1, (size_t)E * 2 * I * H, l), E, 2 * I, H, true, GPTOSS_PACK_GLU, next_seed(), STD);
+    w.b1 = b.upload_f32(at(b1, (size_t)E * 2 * I, l), (size_t)E * 2 * I, next_seed(), 0.f, STD);
+    w.w2 = b.upload_matrices(at(w2, (size_t)E * H * I, l), E, H, I, true, 0, next_seed(), STD);
+    w.b2 = b.upload_f32(at(b2, (size_t)E * H, l), (size_t)E * H, next_seed(), 0.f, STD);
+    // even layers keep only the sliding window (ring buffer), odd layers the whole context
+    // (reference run.cpp:582, getp-csrc/src/alloc.cpp:245-250)
+    const bool windowed = W > 0 && (l % 2 == 0);
+    w.window = windowed ? W : 0;
+    w.cache_cap = windowed ? std::min(cap_full, (int)align_up((size_t)W, 64)) : cap_full;
+    size_t cache_elems = (size_t)max_batch * nkv * w.cache_cap * D;
+    w.k_cache = b.alloc<bf16_t>(cache_elems);
+    w.v_cache = b.alloc<bf16_t>(cache_elems);
+    if (b.ok()) {
+      b.hip(hipMemsetAsync(w.k_cache, 0, cache_elems * 2, e->stream), "memset");
+      b.hip(hipMemsetAsync(w.v_cache, 0, cache_elems * 2, e->stream), "memset");
+    }
+  }
+  if (b.stage_f32) (void)hipFree(b.stage_f32);
+  if (b.stage_bf16) (void)hipFree(b.stage_bf16);
+
+  // rotary tables
+  {
+    std::vector<float> cs, sn;
+    rope_tables(c, max_seq, cs, sn);
+    e->cos_t = b.alloc<float>(cs.size());
+    e->sin_t = b.alloc<float>(sn.size());
+    if (b.ok()) {
+      b.hip(hipMemcpy(e->cos_t, cs.data(), cs.size() * 4, hipMemcpyHostToDevice), "H2D");
+      b.hip(hipMemcpy(e->sin_t, sn.data(), sn.size() * 4, hipMemcpyHostToDevice), "H2D");
+    }
+  }
+  // run state
+  const int B = max_batch;
+  e->d_tokens = b.alloc<int>(B);
+  e->d_next = b.alloc<int>(B);
+  e->d_lens = b.alloc<int>(B);
+  e->x = b.alloc<float>((size_t)B * H);
+  e->t = b.alloc<bf16_t>((size_t)B * H);
+  e->qkv = b.alloc<float>((size_t)B * qkv_dim);
+  e->q = b.alloc<float>((size_t)B * nq * D);
+  e->attn_out = b.alloc<bf16_t>((size_t)B * nq * D);
+  e->tb2 = b.alloc<float>((size_t)B * H);
+  e->logits = b.alloc<float>((size_t)B * V);
+  e->moe_ws_bytes = gptoss_moe_workspace_bytes(B, E, k, H, I);
+  e->moe_ws = b.alloc<unsigned char>(e->moe_ws_bytes);
+  e->attn_ws_bytes = std::max<size_t>(256, gptoss_attn_workspace_bytes(B, nq, nkv, D, max_seq));
+  e->attn_ws = b.alloc<unsigned char>(e->attn_ws_bytes);
+  if (b.ok()) b.hip(hipStreamSynchronize(e->stream), "sync");
+  if (!b.ok()) {
+    destroy(e);
+    return b.rc;
+  }
+  *out = e;
+  return GPTOSS_OK;
+}
+
+extern "C" void gptoss_engine_destroy(gptoss_engine *e) { destroy(e); }
+
+extern "C" int gptoss_engine_step(gptoss_engine *e, const int *host_tokens, int pos, int B, int *host_next) {
+  GPTOSS_REQUIRE(e && host_tokens && host_next, GPTOSS_ERR_NULL, "engine_step: null pointer");
+  GPTOSS_REQUIRE(B >= 1 && B <= e->max_batch, GPTOSS_ERR_DIM, "engine_step: batch %d outside 1..%d", B, e->max_batch);
+  GPTOSS_REQUIRE(pos >= 0 && pos < e->max_seq, GPTOSS_ERR_STATE, "engine_step: position %d outside 0..%d", pos, e->max_seq - 1);
+  const gptoss_config &c = e->cfg;
+  const int H = c.hidden_dim, V = c.vocab_size, L = c.n_layers, E = c.n_experts, k = c.experts_per_token;
+  const int D = c.head_dim, nq = c.n_attn_heads, nkv = c.n_kv_heads, I = c.intermediate_dim;
+  const int qkv_dim = (nq + 2 * nkv) * D;
+  hipStream_t s = e->stream;
+  int rc;
+#define STEP(call)                   \
+  do {                               \
+    rc = (call);                     \
+    if (rc != GPTOSS_OK) return rc;  \
+  } while (0)
+
+  memcpy(e->h_tokens, host_tokens, sizeof(int) * B);
+  GPTOSS_HIP(hipMemcpyAsync(e->d_tokens, e->h_tokens, sizeof(int) * B, hipMemcpyHostToDevice, s));
+  STEP(run_fill_int(e->d_lens, B, pos + 1, s));
+  STEP(run_embedding(e->embedding, e->d_tokens, e->x, B, H, V, s));
+  for (int l = 0; l < L; l++) {
+    const LayerWeights &w = e->layers[l];
+    if (l == 0) STEP(run_rmsnorm(e->x, nullptr, w.attn_norm, e->t, nullptr, B, H, s));
+    STEP(dense_gemm(e->t, w.w_qkv, w.b_qkv, e->qkv, EPI_F32, B, qkv_dim, H, s));
+    STEP(run_rope_store(e->qkv, e->q, w.k_cache, w.v_cache, e->cos_t, e->sin_t, B, nq, nkv, D,
+                        w.cache_cap, pos, s));
+    STEP(gptoss_attn_decode(e->q, w.k_cache, w.v_cache, e->d_lens, w.sinks, e->attn_out, B, nq, nkv, D,
+                            w.cache_cap, w.window, pos + 1, e->attn_ws, e->attn_ws_bytes, s));
+    STEP(dense_gemm(e->attn_out, w.w_o, w.b_o, e->tb2, EPI_F32, B, H, nq * D, s));
+    // x += attention branch, then the ffn norm (model.cpp:66)
+    STEP(run_rmsnorm(e->x, e->tb2, w.mlp_norm, e->t, nullptr, B, H, s));
+    gptoss_moe_weights mw;
+    mw.n_experts = E;
+    mw.top_k = k;
+    mw.hidden = H;
+    mw.intermediate = I;
+    mw.swiglu_limit = c.swiglu_limit;
+    mw.w_router = w.w_router;
+    mw.b_router = w.b_router;
+    mw.w1 = w.w1;
+    mw.b1 = w.b1;
+    mw.w2 = w.w2;
+    mw.b2 = w.b2;
+    // x += MoE branch (the combine kernel adds into the residual stream, model.cpp:121-131)
+    STEP(gptoss_moe_forward(&mw, e->t, B, e->x, 1, e->moe_ws, e->moe_ws_bytes, s));
+    // next layer's attention norm, or the final norm
+    const float *nw = (l + 1 < L) ? e->layers[l + 1].attn_norm : e->final_norm;
+    STEP(run_rmsnorm(e->x, nullptr, nw, e->t, nullptr, B, H, s));
+  }
+  STEP(dense_gemm(e->t, e->unembedding, nullptr, e->logits, EPI_F32, B, V, H, s));
+  STEP(run_argmax(e->logits, e->d_next, B, V, s));
+  GPTOSS_HIP(hipMemcpyAsync(e->h_next, e->d_next, sizeof(int) * B, hipMemcpyDeviceToHost, s));
+  GPTOSS_HIP(hipStreamSynchronize(s));
+  memcpy(host_next, e->h_next, sizeof(int) * B);
+#undef STEP
+  return GPTOSS_OK;
+}
+
+extern "C" int gptoss_engine_generate(gptoss_engine *e, const int *host_prompts, const int *host_n_prompt,
+                                      int prompt_stride, int n_req, int max_seq_len, int *host_out,
+                                      long long *n_generated) {
+  GPTOSS_REQUIRE(e && host_prompts && host_n_prompt && host_out, GPTOSS_ERR_NULL, "engine_generate: null pointer");
+  GPTOSS_REQUIRE(n_req >= 0 && prompt_stride >= 1 && max_seq_len >= 1 && max_seq_len <= e->max_seq + 1,
+                 GPTOSS_ERR_DIM, "engine_generate: max_seq_len %d needs an engine with max_seq >= %d",
+                 max_seq_len, max_seq_len - 1);
+  long long total = 0;
+  for (int r = 0; r < n_req; r++)
+    GPTOSS_REQUIRE(host_n_prompt[r] >= 1 && host_n_prompt[r] <= prompt_stride, GPTOSS_ERR_DIM,
+                   "engine_generate: request %d has %d prompt tokens", r, host_n_prompt[r]);
+  // requests are served in batches of max_batch, all sequences of a batch in lock step
+  // (getp_run_submit.cpp:13-87)
+  for (int r0 = 0; r0 < n_req; r0 += e->max_batch) {
+    const int B = std::min(e->max_batch, n_req - r0);
+    std::vector<int> cur_tok(B), cur_pos(B, 0), next(B);
+    std::vector<char> active(B, 1);
+    int active_count = B;
+    for (int i = 0; i < B; i++) cur_tok[i] = host_prompts[(size_t)(r0 + i) * prompt_stride];
+    for (int pos = 0; pos < max_seq_len - 1 && active_count > 0; pos++) {
+      int rc = gptoss_engine_step(e, cur_tok.data(), pos, B, next.data());
+      if (rc != GPTOSS_OK) return rc;
+      for (int i = 0; i < B; i++) {
+        if (!active[i]) continue;
+        const int *pt = host_prompts + (size_t)(r0 + i) * prompt_stride;
+        const int np = host_n_prompt[r0 + i];
+        int *o = host_out + (size_t)(r0 + i) * (max_seq_len + 1);
+        int nt = next[i];
+        if (cur_pos[i] < np - 1) nt = pt[cur_pos[i] + 1];
+        else o[cur_pos[i] - (np - 1)] = nt;
+        if (nt == 199999 || nt == 200002) {
+          active[i] = 0;
+          active_count--;
+        }
+        cur_tok[i] = nt;
+        cur_pos[i]++;
+      }
+    }
+    for (int i = 0; i < B; i++) {
+      int generated_len = cur_pos[i] - host_n_prompt[r0 + i];
+      if (generated_len < 0) generated_len = 0;
+      host_out[(size_t)(r0 + i) * (max_seq_len + 1) + generated_len + 1] = -1;
+      total += generated_len + 1;
+    }
+  }
+  if (n_generated) *n_generated = total;
+  return GPTOSS_OK;
+}
+
+// Device views for tests and tracing: logits of the last step [B,V] and the residual stream.
+extern "C" int gptoss_engine_debug_views(gptoss_engine *e, float **logits, float **x, size_t *device_bytes) {
+  GPTOSS_REQUIRE(e, GPTOSS_ERR_NULL, "engine_debug_views: null engine");
+  if (logits) *logits = e->logits;
+  if (x) *x = e->x;
+  if (device_bytes) *device_bytes = e->device_bytes;
+  return GPTOSS_OK;
+}

@@ -1,0 +1,235 @@
+// Small memory-bound kernels around the two hot ops of a decode step: embedding gather, RMSNorm
+// (optionally fused with the residual add), q/k/v split + rotary embedding + KV-cache store, row
+// arg-max, dtype conversion and on-device synthetic weight generation.
+#include "common.hpp"
+#include "glue.hpp"
+
+namespace gptoss {
+
+// x[b,:] = embedding[token[b],:]   (bf16 table -> fp32 residual stream)
+// reference: embedding_lookup_kernel, layer_hip_batch.cpp:199-214
+__global__ __launch_bounds__(256) void embedding_kernel(const bf16_t *__restrict__ table,
+                                                        const int *__restrict__ tokens,
+                                                        float *__restrict__ x, int H, int V) {
+  const int b = blockIdx.x;
+  int tok = tokens[b];
+  tok = min(max(tok, 0), V - 1);
+  const bf16_t *row = table + (size_t)tok * H;
+  for (int h = threadIdx.x; h < H; h += 256) x[(size_t)b * H + h] = bf16_to_f32(row[h]);
+}
+
+// RMSNorm with the arithmetic of run.cpp:304-317: sum of squares accumulated in double from
+// float products, eps added after the mean, 1/sqrtf in float, scale applied in double and
+// rounded once.  If residual != nullptr, x += residual first (in place), as
+// residual_rmsnorm_bf16_kernel does (layer_hip_batch.cpp:94-155).
+// Outputs: t_bf16 (always) and t_f32 (optional full-precision copy).
+__global__ __launch_bounds__(256) void rmsnorm_kernel(float *__restrict__ x,
+                                                      const float *__restrict__ residual,
+                                                      const float *__restrict__ weight,
+                                                      bf16_t *__restrict__ t_bf16,
+                                                      float *__restrict__ t_f32, int H) {
+  __shared__ double red[4];
+  const int b = blockIdx.x;
+  float *xr = x + (size_t)b * H;
+  double ss = 0.0;
+  for (int h = threadIdx.x; h < H; h += 256) {
+    float v = xr[h];
+    if (residual) {
+      v = __fadd_rn(v, residual[(size_t)b * H + h]);
+      xr[h] = v;
+    }
+    ss += (double)__fmul_rn(v, v);
+  }
+  for (int m = 32; m >= 1; m >>= 1) ss += __shfl_xor(ss, m, 64);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
+  __syncthreads();
+  ss = red[0] + red[1] + red[2] + red[3];
+  ss /= H;
+  ss += 1e-5f;
+  const double inv = (double)(1.0f / sqrtf((float)ss));
+  for (int h = threadIdx.x; h < H; h += 256) {
+    float o = (float)((double)weight[h] * (inv * (double)xr[h]));
+    t_bf16[(size_t)b * H + h] = f32_to_bf16(o);
+    if (t_f32) t_f32[(size_t)b * H + h] = o;
+  }
+}
+
+// Split the fused qkv row, rotate q and k (half-split pairs i, i+D/2; run.cpp:480-499), write q
+// (fp32) and store k, v as bf16 into this layer's cache slot pos % cap.
+// reference: qkv_split_rope_store_kernel, layer_hip_batch.cpp:686-776
+__global__ __launch_bounds__(256) void rope_store_kernel(const float *__restrict__ qkv,
+                                                         float *__restrict__ q_out,
+                                                         bf16_t *__restrict__ kc, bf16_t *__restrict__ vc,
+                                                         const float *__restrict__ cos_t,
+                                                         const float *__restrict__ sin_t, int n_q,
+                                                         int n_kv, int D, int cap, int pos) {
+  const int b = blockIdx.x;
+  const int half = D >> 1;
+  const int q_dim = n_q * D, kv_dim = n_kv * D;
+  const float *row = qkv + (size_t)b * (q_dim + 2 * kv_dim);
+  const float *cs = cos_t + (size_t)pos * half, *sn = sin_t + (size_t)pos * half;
+  const int slot = pos % cap;
+  for (int p = threadIdx.x; p < n_q * half; p += 256) {
+    int h = p / half, j = p - h * half;
+    float x1 = row[h * D + j], x2 = row[h * D + half + j];
+    float c = cs[j], s = sn[j];
+    q_out[(size_t)b * q_dim + h * D + j] = __fsub_rn(__fmul_rn(x1, c), __fmul_rn(x2, s));
+    q_out[(size_t)b * q_dim + h * D + half + j] = __fadd_rn(__fmul_rn(x2, c), __fmul_rn(x1, s));
+  }
+  for (int p = threadIdx.x; p < n_kv * half; p += 256) {
+    int g = p / half, j = p - g * half;
+    float x1 = row[q_dim + g * D + j], x2 = row[q_dim + g * D + half + j];
+    float c = cs[j], s = sn[j];
+    size_t base = ((size_t)(b * n_kv + g) * cap + slot) * D;
+    kc[base + j] = f32_to_bf16(__fsub_rn(__fmul_rn(x1, c), __fmul_rn(x2, s)));
+    kc[base + half + j] = f32_to_bf16(__fadd_rn(__fmul_rn(x2, c), __fmul_rn(x1, s)));
+  }
+  for (int p = threadIdx.x; p < kv_dim; p += 256) {
+    int g = p / D, d = p - g * D;
+    size_t base = ((size_t)(b * n_kv + g) * cap) * D;
+    int tt = slot & 31, within = tt & 15;
+    int lane = (within >> 2) * 16 + (d & 15);
+    int j = (tt >> 4) * 4 + (within & 3);
+    vc[base + ((size_t)(slot >> 5) * (D / 16) + (d >> 4)) * 512 + lane * 8 + j] =
+        f32_to_bf16(row[q_dim + kv_dim + p]);
+  }
+}
+
+// ids[b] = arg max over logits[b,:], lowest index among equal maxima (run.cpp:739-750).
+// reference: max_kernel_gpu_v2, layer_hip_batch.cpp:1542-1597
+__global__ __launch_bounds__(1024) void argmax_kernel(const float *__restrict__ logits,
+                                                      int *__restrict__ ids, int V) {
+  __shared__ float sv[16];
+  __shared__ int si[16];
+  const int b = blockIdx.x;
+  const float *row = logits + (size_t)b * V;
+  float bv = -INFINITY;
+  int bi = 0x7fffffff;
+  for (int i = threadIdx.x * 4; i < V; i += 1024 * 4) {
+    if (i + 3 < V) {
+      f32x4 v = *reinterpret_cast<const f32x4 *>(row + i);
+#pragma unroll
+      for (int q = 0; q < 4; q++)
+        if (v[q] > bv || bi == 0x7fffffff) { bv = v[q]; bi = i + q; }
+    } else {
+      for (int q = 0; q < 4 && i + q < V; q++)
+        if (row[i + q] > bv || bi == 0x7fffffff) { bv = row[i + q]; bi = i + q; }
+    }
+  }
+  for (int m = 32; m >= 1; m >>= 1) {
+    float ov = __shfl_xor(bv, m, 64);
+    int oi = __shfl_xor(bi, m, 64);
+    if (oi != 0x7fffffff && (bi == 0x7fffffff || ov > bv || (ov == bv && oi < bi))) { bv = ov; bi = oi; }
+  }
+  if ((threadIdx.x & 63) == 0) { sv[threadIdx.x >> 6] = bv; si[threadIdx.x >> 6] = bi; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < 16; w++)
+      if (si[w] != 0x7fffffff && (bi == 0x7fffffff || sv[w] > bv || (sv[w] == bv && si[w] < bi))) {
+        bv = sv[w];
+        bi = si[w];
+      }
+    ids[b] = (bi == 0x7fffffff) ? 0 : bi;
+  }
+}
+
+__global__ __launch_bounds__(256) void f32_to_bf16_kernel(const float *__restrict__ src,
+                                                          bf16_t *__restrict__ dst, size_t n) {
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256)
+    dst[i] = f32_to_bf16(src[i]);
+}
+
+__global__ __launch_bounds__(256) void fill_int_kernel(int *__restrict__ dst, int n, int value) {
+  int i = blockIdx.x * 256 + threadIdx.x;
+  if (i < n) dst[i] = value;
+}
+
+// N(mean, std) from a counter-based generator (splitmix64 of seed+index, Box-Muller), rounded to
+// bf16 or kept fp32.  Used to build random-init models of sizes whose fp32 file would not fit.
+__device__ __forceinline__ uint64_t splitmix64(uint64_t z) {
+  z += 0x9E3779B97F4A7C15ull;
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  return z ^ (z >> 31);
+}
+
+__device__ __forceinline__ float normal_at(uint64_t seed, uint64_t i) {
+  uint64_t r = splitmix64(seed * 0xD1342543DE82EF95ull + i);
+  float u1 = ((uint32_t)(r >> 40) + 1.0f) * (1.0f / 16777217.0f);  // (0,1]
+  float u2 = (uint32_t)(r & 0xffffffu) * (1.0f / 16777216.0f);
+  return sqrtf(-2.0f * __logf(u1)) * __cosf(6.2831853071795865f * u2);
+}
+
+__global__ __launch_bounds__(256) void synth_normal_bf16_kernel(bf16_t *__restrict__ dst, size_t n,
+                                                                uint64_t seed, float mean, float std) {
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256)
+    dst[i] = f32_to_bf16(mean + std * normal_at(seed, i));
+}
+
+__global__ __launch_bounds__(256) void synth_normal_f32_kernel(float *__restrict__ dst, size_t n,
+                                                               uint64_t seed, float mean, float std) {
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256)
+    dst[i] = bf16_to_f32(f32_to_bf16(mean + std * normal_at(seed, i)));
+}
+
+static inline int grid_for(size_t n) {
+  size_t g = (n + 255) / 256;
+  return (int)(g > 65536 ? 65536 : (g == 0 ? 1 : g));
+}
+
+int run_embedding(const bf16_t *table, const int *tokens, float *x, int B, int H, int V, hipStream_t s) {
+  TraceScope ts("embedding", s);
+  embedding_kernel<<<B, 256, 0, s>>>(table, tokens, x, H, V);
+  GPTOSS_LAUNCH_CHECK("embedding_kernel");
+  return GPTOSS_OK;
+}
+
+int run_rmsnorm(float *x, const float *residual, const float *weight, bf16_t *t_bf16, float *t_f32,
+                int B, int H, hipStream_t s) {
+  TraceScope ts(residual ? "residual_rmsnorm" : "rmsnorm", s);
+  rmsnorm_kernel<<<B, 256, 0, s>>>(x, residual, weight, t_bf16, t_f32, H);
+  GPTOSS_LAUNCH_CHECK("rmsnorm_kernel");
+  return GPTOSS_OK;
+}
+
+int run_rope_store(const float *qkv, float *q_out, bf16_t *kc, bf16_t *vc, const float *cos_t,
+                   const float *sin_t, int B, int n_q, int n_kv, int D, int cap, int pos,
+                   hipStream_t s) {
+  TraceScope ts("rope_store", s);
+  rope_store_kernel<<<B, 256, 0, s>>>(qkv, q_out, kc, vc, cos_t, sin_t, n_q, n_kv, D, cap, pos);
+  GPTOSS_LAUNCH_CHECK("rope_store_kernel");
+  return GPTOSS_OK;
+}
+
+int run_argmax(const float *logits, int *ids, int B, int V, hipStream_t s) {
+  TraceScope ts("argmax", s);
+  argmax_kernel<<<B, 1024, 0, s>>>(logits, ids, V);
+  GPTOSS_LAUNCH_CHECK("argmax_kernel");
+  return GPTOSS_OK;
+}
+
+int run_f32_to_bf16(const float *src, bf16_t *dst, size_t n, hipStream_t s) {
+  f32_to_bf16_kernel<<<grid_for(n), 256, 0, s>>>(src, dst, n);
+  GPTOSS_LAUNCH_CHECK("f32_to_bf16_kernel");
+  return GPTOSS_OK;
+}
+
+int run_fill_int(int *dst, int n, int value, hipStream_t s) {
+  fill_int_kernel<<<cdiv(n, 256), 256, 0, s>>>(dst, n, value);
+  GPTOSS_LAUNCH_CHECK("fill_int_kernel");
+  return GPTOSS_OK;
+}
+
+int run_synth_bf16(bf16_t *dst, size_t n, uint64_t seed, float mean, float std, hipStream_t s) {
+  synth_normal_bf16_kernel<<<grid_for(n), 256, 0, s>>>(dst, n, seed, mean, std);
+  GPTOSS_LAUNCH_CHECK("synth_normal_bf16_kernel");
+  return GPTOSS_OK;
+}
+
+int run_synth_f32(float *dst, size_t n, uint64_t seed, float mean, float std, hipStream_t s) {
+  synth_normal_f32_kernel<<<grid_for(n), 256, 0, s>>>(dst, n, seed, mean, std);
+  GPTOSS_LAUNCH_CHECK("synth_normal_f32_kernel");
+  return GPTOSS_OK;
+}
+
+}  // namespace gptoss

@@ -1,0 +1,20 @@
+// Internal interface of the glue kernels (glue.hip).
+#pragma once
+#include "common.hpp"
+
+namespace gptoss {
+
+int run_embedding(const bf16_t *table, const int *tokens, float *x, int B, int H, int V, hipStream_t s);
+// x (+= residual) -> t_bf16 (and t_f32 when not null); residual may be null
+int run_rmsnorm(float *x, const float *residual, const float *weight, bf16_t *t_bf16, float *t_f32,
+                int B, int H, hipStream_t s);
+int run_rope_store(const float *qkv, float *q_out, bf16_t *kc, bf16_t *vc, const float *cos_t,
+                   const float *sin_t, int B, int n_q, int n_kv, int D, int cap, int pos,
+                   hipStream_t s);
+int run_argmax(const float *logits, int *ids, int B, int V, hipStream_t s);
+int run_f32_to_bf16(const float *src, bf16_t *dst, size_t n, hipStream_t s);
+int run_fill_int(int *dst, int n, int value, hipStream_t s);
+int run_synth_bf16(bf16_t *dst, size_t n, uint64_t seed, float mean, float std, hipStream_t s);
+int run_synth_f32(float *dst, size_t n, uint64_t seed, float mean, float std, hipStream_t s);
+
+}  // namespace gptoss

@@ -77,6 +77,7 @@ SIGNATURES = {
     "gptoss_engine_step": (_i, [_vp, _vp, _i, _i, _vp]),
     "gptoss_engine_generate": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp, C.POINTER(C.c_longlong)]),
     "gptoss_engine_destroy": (None, [_vp]),
+    "gptoss_engine_debug_views": (_i, [_vp, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_sz)]),
 }
 
 _lib = None

@@ -220,3 +220,74 @@ class KernelTrace:
             c, t = agg.get(name, (0, 0.0))
             agg[name] = (c + 1, t + ms)
         return {k: (c, t / c) for k, (c, t) in agg.items()}
+
+
+class Engine:
+    """Single-GPU decode engine over a flat ``.bin`` payload (or synthetic on-device weights)."""
+
+    def __init__(self, cfg, weights_flat=None, max_batch=8, max_seq=64, synthetic=False,
+                 precise=False, seed=0):
+        _need_gpu()
+        import numpy as np
+        self.L = _l.load()
+        self.cfg = cfg
+        self.max_batch, self.max_seq = max_batch, max_seq
+        flags = (_l.ENGINE_SYNTHETIC if synthetic else 0) | (_l.ENGINE_PRECISE if precise else 0)
+        self._cc = _l.Config.from_config(cfg)
+        wp = None
+        if not synthetic:
+            self._w = np.ascontiguousarray(weights_flat, dtype=np.float32)
+            wp = self._w.ctypes.data_as(C.c_void_p)
+        h = C.c_void_p()
+        _l.check(self.L.gptoss_engine_create(C.byref(self._cc), wp, max_batch, max_seq, flags,
+                                             C.c_uint64(seed), C.byref(h)))
+        self._h = h
+
+    def step(self, tokens, pos):
+        import numpy as np
+        tok = np.ascontiguousarray(tokens, dtype=np.int32)
+        nxt = np.empty_like(tok)
+        _l.check(self.L.gptoss_engine_step(self._h, tok.ctypes.data_as(C.c_void_p), int(pos),
+                                           tok.size, nxt.ctypes.data_as(C.c_void_p)))
+        return nxt
+
+    def generate(self, prompts, max_seq_len, n_prompt=None):
+        import numpy as np
+        prompts = np.ascontiguousarray(prompts, dtype=np.int32)
+        n_req, stride = prompts.shape
+        npr = np.full(n_req, stride, np.int32) if n_prompt is None else \
+            np.ascontiguousarray(n_prompt, dtype=np.int32)
+        out = np.zeros((n_req, max_seq_len + 1), np.int32)
+        n = C.c_longlong(0)
+        _l.check(self.L.gptoss_engine_generate(self._h, prompts.ctypes.data_as(C.c_void_p),
+                                               npr.ctypes.data_as(C.c_void_p), stride, n_req,
+                                               max_seq_len, out.ctypes.data_as(C.c_void_p),
+                                               C.byref(n)))
+        return out, int(n.value)
+
+    def last_logits(self, B):
+        """fp32 [B, vocab] logits of the last step (copied to the host)."""
+        lp, xp, nb = C.c_void_p(), C.c_void_p(), C.c_size_t()
+        _l.check(self.L.gptoss_engine_debug_views(self._h, C.byref(lp), C.byref(xp), C.byref(nb)))
+        V = self.cfg.vocab_size
+        host = torch.empty(B, V, dtype=torch.float32)
+        torch.cuda.synchronize()
+        # a plain device-to-host copy of memory the engine owns
+        rt = C.CDLL("libamdhip64.so")
+        rc = rt.hipMemcpy(C.c_void_p(host.data_ptr()), lp, C.c_size_t(B * V * 4), 2)
+        if rc != 0:
+            raise RuntimeError(f"hipMemcpy failed: {rc}")
+        return host.numpy()
+
+    def device_bytes(self):
+        nb = C.c_size_t()
+        _l.check(self.L.gptoss_engine_debug_views(self._h, None, None, C.byref(nb)))
+        return nb.value
+
+    def close(self):
+        if getattr(self, "_h", None):
+            self.L.gptoss_engine_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        self.close()

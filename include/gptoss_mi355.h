@@ -224,6 +224,11 @@ int gptoss_engine_generate(gptoss_engine *e, const int *host_prompts, const int 
 
 void gptoss_engine_destroy(gptoss_engine *e);
 
+/* Device views for tests and tracing (the counterpart of the reference's Tensor::printDebug,
+ * getp-csrc/src/tensor.cpp:158-172): logits fp32 [B,vocab] and residual stream fp32 [B,hidden] of
+ * the last step, and the bytes of device memory the engine holds.  Outputs may be NULL. */
+int gptoss_engine_debug_views(gptoss_engine *e, float **logits, float **x, size_t *device_bytes);
+
 #ifdef __cplusplus
 }
 #endif

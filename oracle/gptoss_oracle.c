@@ -393,6 +393,7 @@ typedef struct {
   float *cos_t, *sin_t;           /* [seq_len, D/2] */
   int stage;
   float min_router_gap; /* smallest (k-th - (k+1)-th) router score seen by orc_forward */
+  float last_router_gap; /* the same over the layers of the last orc_forward call only */
 } OrcModel;
 
 long long orc_weight_floats(const OrcConfig *c) {
@@ -463,6 +464,7 @@ void orc_model_destroy(OrcModel *m) {
 float *orc_model_logits(OrcModel *m) { return m->logits; }
 float *orc_model_x(OrcModel *m) { return m->x; }
 float orc_model_min_router_gap(OrcModel *m) { return m->min_router_gap; }
+float orc_model_last_router_gap(OrcModel *m) { return m->last_router_gap; }
 
 static void round_vec(float *x, long long n) {
   for (long long i = 0; i < n; i++) x[i] = bf16_round(x[i]);
@@ -496,6 +498,7 @@ float *orc_forward(OrcModel *m, int token, int pos) {
   int S = p->seq_len;
   int stage = m->stage;
 
+  m->last_router_gap = INFINITY;
   memcpy(x, m->emb + 1ll * token * hidden_dim, hidden_dim * sizeof(float));
 
   for (long long l = 0; l < p->n_layers; l++) {
@@ -569,6 +572,7 @@ float *orc_forward(OrcModel *m, int token, int pos) {
         if (!picked && m->score[i] > next) next = m->score[i];
       }
       if (kth - next < m->min_router_gap) m->min_router_gap = kth - next;
+      if (kth - next < m->last_router_gap) m->last_router_gap = kth - next;
     }
     memset(m->e_agg, 0, hidden_dim * sizeof(float));
     for (int e = 0; e < E; e++) {

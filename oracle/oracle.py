@@ -72,6 +72,8 @@ def lib():
         L.orc_model_create.restype = C.c_void_p
         L.orc_forward.restype = C.POINTER(C.c_float)
         L.orc_model_x.restype = C.POINTER(C.c_float)
+        L.orc_model_last_router_gap.restype = C.c_float
+        L.orc_model_min_router_gap.restype = C.c_float
         _lib = L
     return _lib
 
@@ -218,10 +220,15 @@ class Model:
         p = lib().orc_model_x(self._h)
         return np.ctypeslib.as_array(p, shape=(self.cfg.hidden_dim,)).copy()
 
+    def last_router_gap(self):
+        """Smallest gap between the k-th and (k+1)-th router score over the layers of the last
+        forward call: how close that call came to picking a different expert."""
+        return float(lib().orc_model_last_router_gap(self._h))
+
     def close(self):
-        if self._h:
-            lib().orc_model_destroy(self._h)
-            self._h = None
+        if self._h and _lib is not None:
+            _lib.orc_model_destroy(self._h)
+        self._h = None
 
     def __del__(self):
         self.close()
