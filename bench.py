@@ -151,6 +151,45 @@ def bench_attn(ops, torch, steps, warmup):
     return res
 
 
+def bench_e2e(ops, torch, n_req=1024, n_prompt=128, n_decode=256):
+    """configs[3]: full GPT-OSS-20B shape, random-init bf16 weights generated on the device,
+    1024 prompts of 128 random ids forced token by token, then 256 greedy decode steps, all
+    sequences in lock step (the reference's getp scheduling)."""
+    import numpy as np
+    synth = importlib.import_module("gpt-oss-team01_amd.synth")
+    cfg = synth.gptoss20b_config(max_seq_len=n_prompt + n_decode)
+    t0 = time.perf_counter()
+    eng = ops.Engine(cfg, None, max_batch=n_req, max_seq=n_prompt + n_decode, synthetic=True, seed=1)
+    t_create = time.perf_counter() - t0
+    rng = np.random.default_rng(3)
+    prompts = rng.integers(0, cfg.vocab_size, size=(n_req, n_prompt), dtype=np.int32)
+    tok = prompts[:, 0].copy()
+    eng.step(tok, 0)                                   # warm-up of every kernel
+    t0 = time.perf_counter()
+    for pos in range(n_prompt - 1):                    # forced prompt positions
+        eng.step(prompts[:, pos], pos)
+    t_prompt = time.perf_counter() - t0
+    tok = prompts[:, n_prompt - 1].copy()
+    t0 = time.perf_counter()
+    for pos in range(n_prompt - 1, n_prompt - 1 + n_decode):
+        tok = eng.step(tok, pos)
+    t_decode = time.perf_counter() - t0
+    trace = ops.KernelTrace(capacity=2048)
+    with trace:
+        eng.step(tok, n_prompt + n_decode - 1)
+    kern = trace.summary()
+    dev_gb = eng.device_bytes() / 1e9
+    eng.close()
+    return {"decode_tok_s": round(n_req * n_decode / t_decode, 1),
+            "decode_ms_per_step": round(t_decode / n_decode * 1e3, 3),
+            "prompt_tok_s": round(n_req * (n_prompt - 1) / t_prompt, 1),
+            "total_tok_s": round(n_req * (n_prompt - 1 + n_decode) / (t_prompt + t_decode), 1),
+            "engine_create_s": round(t_create, 1), "device_gb": round(dev_gb, 1),
+            "last_step_kernels_us": {k: [c, round(ms * c * 1e3, 1)] for k, (c, ms) in kern.items()},
+            "config": "24 blocks, hidden 2880, 64q/8kv heads x 64, 32 experts top-4, vocab 201088, "
+                      "window 128 on even layers; 1024 seqs x (128 forced + 256 decoded)"}
+
+
 def main():
     args = parse()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -186,6 +225,10 @@ def main():
              "gemm1_tflops": round(moe["gemm1_flops"] / moe["gemm1_ms"] / 1e9, 1)}
     if not args.no_attn:
         extra["decode_attn"] = bench_attn(ops, torch, max(10, args.steps // 2), args.warmup)
+
+    if not args.no_e2e:
+        torch.cuda.empty_cache()
+        extra["e2e_20b"] = bench_e2e(ops, torch)
 
     achieved = moe["gemm1_bytes"] / moe["gemm1_ms"] / 1e6
     line = {

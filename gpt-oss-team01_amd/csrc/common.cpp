@@ -32,13 +32,13 @@ const char *last_error() { return g_last_error; }
 struct TraceState {
   hipEvent_t *start = nullptr, *stop = nullptr;
   int capacity = 0, count = 0;
-  const char *names[256];
+  const char *names[4096];
 };
 static thread_local TraceState g_trace;
 
 TraceScope::TraceScope(const char *name, hipStream_t s) : slot(-1), stream(s) {
   TraceState &t = g_trace;
-  if (t.start == nullptr || t.count >= t.capacity || t.count >= 256) return;
+  if (t.start == nullptr || t.count >= t.capacity || t.count >= 4096) return;
   slot = t.count++;
   t.names[slot] = name;
   (void)hipEventRecord(t.start[slot], stream);

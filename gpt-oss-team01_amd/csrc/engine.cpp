@@ -188,7 +188,10 @@ int dense_gemm(const bf16_t *A, const bf16_t *W, const float *bias, void *out, i
   g.N = N;
   g.K = K;
   g.n_col_tiles = cdiv(N, 256);
-  int rpt = B > 128 ? 256 : (B > 64 ? 128 : (B > 32 ? 64 : 32));
+  // largest row tile that still gives the 256 CUs at least one workgroup each; the weights of
+  // these GEMMs are small enough to be re-read from L2 by the extra row tiles
+  int rpt = 256;
+  while (rpt > 32 && (rpt / 2 >= B || cdiv(B, rpt) * g.n_col_tiles < 256)) rpt /= 2;
   return run_gemm(g, false, epi, rpt, cdiv(B, rpt), s);
 }
 

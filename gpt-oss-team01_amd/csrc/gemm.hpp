@@ -10,7 +10,8 @@ struct GemmParams {
   const bf16_t *A;     // activations, row-major [*, K]
   const int *row_ids;  // gather: sorted pair ids (row of A = id / top_k); else unused
   int top_k;
-  const bf16_t *W;     // packed weights, per-matrix stride N*K
+  const bf16_t *W;     // packed weights, per-matrix stride N*K (or MXFP4 bytes when w_mxfp4)
+  int w_mxfp4;         // W holds gptoss_pack_mxfp4 output
   const float *bias;   // [n_mat, N] or nullptr
   void *out;           // EPI_F32: float [*, N]; EPI_SWIGLU: bf16 [*, N/2]; EPI_BF16: bf16 [*, N]
   const int *tiles;    // {n_tiles, (mat,row0,rows)*} or nullptr for a dense problem

@@ -34,7 +34,44 @@ constexpr int BN = 256;           // virtual columns per workgroup (4 waves x 64
 // One (row tile, column tile) work item with a compile-time number of 32-row blocks, so every
 // loop below is fully unrolled and every global load is unconditional (the wait counters the
 // compiler derives stay exact and the prefetches stay in flight across iterations).
-template <int MB, bool GATHER, int EPI>
+// MXFP4 operand expansion.  One dword holds the lane's 8 e2m1 codes of a k-step (element j < 4 in
+// the low nibble of byte j, element j >= 4 in the high nibble of byte j-4).  tab[] holds the eight
+// positive bf16 magnitudes already multiplied by the block's power-of-two scale, as byte tables
+// for v_perm_b32: tab[0]/tab[1] = low bytes of entries 0-3 / 4-7, tab[2]/tab[3] = high bytes.
+struct Fp4Table {
+  uint32_t lo_a, lo_b, hi_a, hi_b;
+};
+
+__device__ __forceinline__ Fp4Table fp4_table(uint32_t e8m0) {
+  // bf16 bit patterns of 0, .5 | 1, 1.5 | 2, 3 | 4, 6 as pairs; the exponent field starts at bit 7
+  // d * 0x00800080 adds d to both exponent fields: for negative d the borrow out of the low half
+  // is undone by the carry of the low-half addition below
+  const uint32_t dd = (e8m0 - 127u) * 0x00800080u;
+  const uint32_t t01 = 0x3F000000u + ((e8m0 - 127u) << 23);  // entry 0 stays +0
+  const uint32_t t23 = 0x3FC03F80u + dd;
+  const uint32_t t45 = 0x40404000u + dd;
+  const uint32_t t67 = 0x40C04080u + dd;
+  Fp4Table t;
+  // v_perm_b32(S0, S1, sel): selector values 0-3 pick bytes of S1, 4-7 bytes of S0
+  t.lo_a = __builtin_amdgcn_perm(t23, t01, 0x06040200u);
+  t.hi_a = __builtin_amdgcn_perm(t23, t01, 0x07050301u);
+  t.lo_b = __builtin_amdgcn_perm(t67, t45, 0x06040200u);
+  t.hi_b = __builtin_amdgcn_perm(t67, t45, 0x07050301u);
+  return t;
+}
+
+__device__ __forceinline__ u32x4 fp4_expand(uint32_t w, const Fp4Table &t) {
+  const uint32_t m_lo = w & 0x07070707u, m_hi = (w >> 4) & 0x07070707u;
+  uint32_t l0 = __builtin_amdgcn_perm(t.lo_b, t.lo_a, m_lo);
+  uint32_t h0 = __builtin_amdgcn_perm(t.hi_b, t.hi_a, m_lo) | ((w << 4) & 0x80808080u);
+  uint32_t l1 = __builtin_amdgcn_perm(t.lo_b, t.lo_a, m_hi);
+  uint32_t h1 = __builtin_amdgcn_perm(t.hi_b, t.hi_a, m_hi) | (w & 0x80808080u);
+  // interleave low and high bytes into bf16 pairs: elements 0,1 | 2,3 | 4,5 | 6,7
+  return u32x4{__builtin_amdgcn_perm(h0, l0, 0x05010400u), __builtin_amdgcn_perm(h0, l0, 0x07030602u),
+               __builtin_amdgcn_perm(h1, l1, 0x05010400u), __builtin_amdgcn_perm(h1, l1, 0x07030602u)};
+}
+
+template <int MB, bool GATHER, int EPI, bool FP4>
 __device__ __forceinline__ void gemm_tile(const GemmParams &p, bf16_t *lds, int lds_stage, int mat,
                                           int row0, int rows, int ct) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -73,17 +110,39 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, bf16_t *lds, int 
   };
 
   // ---- B: two fragment streams per wave, three slabs in the register ring ---------------------
-  const bf16_t *wbase = p.W + (size_t)mat * N * K + ((size_t)(n0 >> 5) * ksteps * 64 + lane) * 8;
-  const size_t frag_stride = (size_t)ksteps * 512;  // elements between adjacent 32-column blocks
-  u32x4 breg[3][2][4];
+  // bf16: 4 x 16 bytes per fragment and slab.  MXFP4: 16 bytes of codes (the lane's 8 codes of each
+  // of the 4 k-steps) + 2 scale bytes (one e8m0 per 32 k) per fragment and slab.
+  constexpr int BQ = FP4 ? 1 : 4;
+  const bf16_t *wbase = nullptr;
+  const unsigned char *cbase = nullptr, *sbase = nullptr;
+  size_t frag_stride = 0, sfrag_stride = 0;
+  if (FP4) {
+    const size_t mat_bytes = (size_t)N * K / 2 + (size_t)N * K / 32;
+    const unsigned char *mb_ = reinterpret_cast<const unsigned char *>(p.W) + (size_t)mat * mat_bytes;
+    cbase = mb_ + ((size_t)(n0 >> 5) * nslab * 64 + lane) * 16;
+    sbase = mb_ + (size_t)N * K / 2 + ((size_t)(n0 >> 5) * nslab * 32 + (lane & 31)) * 2;
+    frag_stride = (size_t)nslab * 1024;
+    sfrag_stride = (size_t)nslab * 64;
+  } else {
+    wbase = p.W + (size_t)mat * N * K + ((size_t)(n0 >> 5) * ksteps * 64 + lane) * 8;
+    frag_stride = (size_t)ksteps * 512;  // elements between adjacent 32-column blocks
+  }
+  u32x4 breg[3][2][BQ];
+  uint32_t sreg[3][2];
   auto load_b = [&](int s, auto ring) {
     constexpr int R = decltype(ring)::value;
 #pragma unroll
-    for (int f = 0; f < 2; f++)
+    for (int f = 0; f < 2; f++) {
+      if (FP4) {
+        breg[R][f][0] = *reinterpret_cast<const u32x4 *>(cbase + f * frag_stride + (size_t)s * 1024);
+        sreg[R][f] = *reinterpret_cast<const unsigned short *>(sbase + f * sfrag_stride + (size_t)s * 64);
+      } else {
 #pragma unroll
-      for (int kk = 0; kk < 4; kk++)
-        breg[R][f][kk] = *reinterpret_cast<const u32x4 *>(wbase + f * frag_stride +
-                                                          (size_t)(s * 4 + kk) * 512);
+        for (int kk = 0; kk < 4; kk++)
+          breg[R][f][kk % BQ] = *reinterpret_cast<const u32x4 *>(wbase + f * frag_stride +
+                                                                 (size_t)(s * 4 + kk) * 512);
+      }
+    }
   };
 
   f32x16 acc[MB][2];
@@ -98,9 +157,24 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, bf16_t *lds, int 
   auto compute = [&](int stage, auto ring) {
     constexpr int R = decltype(ring)::value;
     const bf16_t *base = a_src + stage * lds_stage;
+    Fp4Table tab[2][2];
+    if (FP4) {
+#pragma unroll
+      for (int f = 0; f < 2; f++) {
+        tab[f][0] = fp4_table(sreg[R][f] & 0xffu);
+        tab[f][1] = fp4_table((sreg[R][f] >> 8) & 0xffu);
+      }
+    }
 #pragma unroll
     for (int kk = 0; kk < 4; kk++) {
-      bf16x8 b0 = as_bf16x8(breg[R][0][kk]), b1 = as_bf16x8(breg[R][1][kk]);
+      bf16x8 b0, b1;
+      if (FP4) {
+        b0 = as_bf16x8(fp4_expand(breg[R][0][0][kk], tab[0][kk >> 1]));
+        b1 = as_bf16x8(fp4_expand(breg[R][1][0][kk], tab[1][kk >> 1]));
+      } else {
+        b0 = as_bf16x8(breg[R][0][kk % BQ]);
+        b1 = as_bf16x8(breg[R][1][kk % BQ]);
+      }
 #pragma unroll
       for (int i = 0; i < MB; i++) {
         bf16x8 a = as_bf16x8(*reinterpret_cast<const u32x4 *>(base + i * 32 * LDS_ROW + kk * 16));
@@ -194,7 +268,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, bf16_t *lds, int 
   }
 }
 
-template <int MBMAX, bool GATHER, int EPI>
+template <int MBMAX, bool GATHER, int EPI, bool FP4>
 __global__ __launch_bounds__(GEMM_THREADS) void grouped_gemm_kernel(GemmParams p) {
   constexpr int BM = MBMAX * 32;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
@@ -223,18 +297,18 @@ __global__ __launch_bounds__(GEMM_THREADS) void grouped_gemm_kernel(GemmParams p
   }
   const int mb = (rows + 31) >> 5;
   if (MBMAX >= 8 && mb > 6) {
-    if (mb == 8) gemm_tile<(MBMAX >= 8 ? 8 : MBMAX), GATHER, EPI>(p, lds, STAGE, mat, row0, rows, ct);
-    else gemm_tile<(MBMAX >= 8 ? 7 : MBMAX), GATHER, EPI>(p, lds, STAGE, mat, row0, rows, ct);
+    if (mb == 8) gemm_tile<(MBMAX >= 8 ? 8 : MBMAX), GATHER, EPI, FP4>(p, lds, STAGE, mat, row0, rows, ct);
+    else gemm_tile<(MBMAX >= 8 ? 7 : MBMAX), GATHER, EPI, FP4>(p, lds, STAGE, mat, row0, rows, ct);
   } else if (MBMAX >= 8 && mb > 4) {
-    if (mb == 6) gemm_tile<(MBMAX >= 8 ? 6 : MBMAX), GATHER, EPI>(p, lds, STAGE, mat, row0, rows, ct);
-    else gemm_tile<(MBMAX >= 8 ? 5 : MBMAX), GATHER, EPI>(p, lds, STAGE, mat, row0, rows, ct);
+    if (mb == 6) gemm_tile<(MBMAX >= 8 ? 6 : MBMAX), GATHER, EPI, FP4>(p, lds, STAGE, mat, row0, rows, ct);
+    else gemm_tile<(MBMAX >= 8 ? 5 : MBMAX), GATHER, EPI, FP4>(p, lds, STAGE, mat, row0, rows, ct);
   } else if (MBMAX >= 4 && mb > 2) {
-    if (mb == 4) gemm_tile<(MBMAX >= 4 ? 4 : MBMAX), GATHER, EPI>(p, lds, STAGE, mat, row0, rows, ct);
-    else gemm_tile<(MBMAX >= 4 ? 3 : MBMAX), GATHER, EPI>(p, lds, STAGE, mat, row0, rows, ct);
+    if (mb == 4) gemm_tile<(MBMAX >= 4 ? 4 : MBMAX), GATHER, EPI, FP4>(p, lds, STAGE, mat, row0, rows, ct);
+    else gemm_tile<(MBMAX >= 4 ? 3 : MBMAX), GATHER, EPI, FP4>(p, lds, STAGE, mat, row0, rows, ct);
   } else if (MBMAX >= 2 && mb == 2) {
-    gemm_tile<(MBMAX >= 2 ? 2 : MBMAX), GATHER, EPI>(p, lds, STAGE, mat, row0, rows, ct);
+    gemm_tile<(MBMAX >= 2 ? 2 : MBMAX), GATHER, EPI, FP4>(p, lds, STAGE, mat, row0, rows, ct);
   } else {
-    gemm_tile<1, GATHER, EPI>(p, lds, STAGE, mat, row0, rows, ct);
+    gemm_tile<1, GATHER, EPI, FP4>(p, lds, STAGE, mat, row0, rows, ct);
   }
 }
 
@@ -316,11 +390,53 @@ __global__ __launch_bounds__(256) void pack_weight_kernel(const SRC *__restrict_
   *dp = u32x4{o[0], o[1], o[2], o[3]};
 }
 
-template <int MB, bool GATHER, int EPI>
+// MXFP4 repack: blocks [n_out, n_in/2] (low nibble = even element) and e8m0 scales [n_out, n_in/32]
+// -> per (32-column block, 64-k slab): 64 lanes x 16 bytes of codes, then 32 x 2 scale bytes.
+__global__ __launch_bounds__(256) void pack_mxfp4_kernel(const unsigned char *__restrict__ blocks,
+                                                         const unsigned char *__restrict__ scales,
+                                                         unsigned char *__restrict__ dst, int n_out,
+                                                         int n_in, int glu) {
+  const int nslab = n_in / 64;
+  const size_t items = (size_t)(n_out / 32) * nslab;          // (column block, slab)
+  const size_t gid = (size_t)blockIdx.x * 256 + threadIdx.x;  // one (item, lane) per thread
+  const size_t item = gid >> 6;
+  const int lane = (int)(gid & 63);
+  const int mat = blockIdx.y;
+  if (item >= items) return;
+  const int nb = (int)(item / nslab), slab = (int)(item - (size_t)nb * nslab);
+  int v = nb * 32 + (lane & 31);
+  int row = v;
+  if (glu) row = 2 * ((v >> 6) * 32 + (v & 31)) + ((v >> 5) & 1);
+  const size_t mat_bytes = (size_t)n_out * n_in / 2 + (size_t)n_out * n_in / 32;
+  const unsigned char *brow = blocks + ((size_t)mat * n_out + row) * (n_in / 2);
+  const unsigned char *srow = scales + ((size_t)mat * n_out + row) * (n_in / 32);
+  unsigned char *md = dst + (size_t)mat * mat_bytes;
+  uint32_t w[4];
+#pragma unroll
+  for (int kk = 0; kk < 4; kk++) {
+    const int k0 = (slab * 4 + kk) * 16 + (lane >> 5) * 8;  // the lane's 8 consecutive k
+    uint32_t src = *reinterpret_cast<const uint32_t *>(brow + k0 / 2);  // nibble j = element k0+j
+    uint32_t o = 0;
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+      uint32_t code = (src >> (4 * j)) & 0xfu;
+      o |= code << ((j < 4) ? (8 * j) : (8 * (j - 4) + 4));
+    }
+    w[kk] = o;
+  }
+  *reinterpret_cast<u32x4 *>(md + (item * 64 + lane) * 16) = u32x4{w[0], w[1], w[2], w[3]};
+  if (lane < 32) {
+    unsigned char *sd = md + (size_t)n_out * n_in / 2 + (item * 32 + lane) * 2;
+    sd[0] = srow[slab * 2];
+    sd[1] = srow[slab * 2 + 1];
+  }
+}
+
+template <int MB, bool GATHER, int EPI, bool FP4 = false>
 static int launch_gemm(const GemmParams &p, int max_tiles, hipStream_t s) {
   static bool attr_done = false;
   size_t smem = (size_t)2 * MB * 32 * LDS_ROW * sizeof(bf16_t);
-  auto kern = grouped_gemm_kernel<MB, GATHER, EPI>;
+  auto kern = grouped_gemm_kernel<MB, GATHER, EPI, FP4>;
   if (!attr_done) {
     GPTOSS_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
@@ -330,7 +446,7 @@ static int launch_gemm(const GemmParams &p, int max_tiles, hipStream_t s) {
   int grid = ((total + 7) / 8) * 8;
   if (grid == 0) return GPTOSS_OK;
   {
-    TraceScope ts(GATHER ? "gemm1_gather_swiglu" : (EPI == EPI_F32 ? "gemm_f32" : (EPI == EPI_BF16 ? "gemm_bf16" : "gemm_swiglu")), s);
+    TraceScope ts(FP4 ? (GATHER ? "gemm1_gather_swiglu_mxfp4" : "gemm_f32_mxfp4") : GATHER ? "gemm1_gather_swiglu" : (EPI == EPI_F32 ? "gemm_f32" : (EPI == EPI_BF16 ? "gemm_bf16" : "gemm_swiglu")), s);
     hipLaunchKernelGGL(kern, dim3(grid), dim3(GEMM_THREADS), smem, s, p);
   }
   GPTOSS_LAUNCH_CHECK("grouped_gemm_kernel");
@@ -341,7 +457,10 @@ static int launch_gemm(const GemmParams &p, int max_tiles, hipStream_t s) {
 int run_gemm(const GemmParams &p, bool gather, int epi, int rows_per_tile, int max_tiles,
              hipStream_t s) {
 #define GPTOSS_GEMM_CASE(MBV)                                                                  \
-  if (rows_per_tile == MBV * 32) {                                                             \
+  if (rows_per_tile == MBV * 32 && p.w_mxfp4) {                                                \
+    if (gather && epi == EPI_SWIGLU) return launch_gemm<MBV, true, EPI_SWIGLU, true>(p, max_tiles, s); \
+    if (!gather && epi == EPI_F32) return launch_gemm<MBV, false, EPI_F32, true>(p, max_tiles, s); \
+  } else if (rows_per_tile == MBV * 32) {                                                      \
     if (gather && epi == EPI_SWIGLU) return launch_gemm<MBV, true, EPI_SWIGLU>(p, max_tiles, s); \
     if (!gather && epi == EPI_F32) return launch_gemm<MBV, false, EPI_F32>(p, max_tiles, s);    \
     if (!gather && epi == EPI_BF16) return launch_gemm<MBV, false, EPI_BF16>(p, max_tiles, s);  \
@@ -393,5 +512,28 @@ extern "C" int gptoss_pack_weight(const void *src, void *dst, int n_mat, int n_o
   else
     pack_weight_kernel<bf16_t><<<grid, 256, 0, s>>>((const bf16_t *)src, (bf16_t *)dst, n_out, n_in, glu);
   GPTOSS_LAUNCH_CHECK("pack_weight_kernel");
+  return GPTOSS_OK;
+}
+
+extern "C" size_t gptoss_packed_mxfp4_bytes(int n_mat, int n_out, int n_in) {
+  if (n_mat <= 0 || n_out <= 0 || n_in <= 0) return 0;
+  return (size_t)n_mat * ((size_t)n_out * n_in / 2 + (size_t)n_out * n_in / 32);
+}
+
+extern "C" int gptoss_pack_mxfp4(const void *blocks, const void *scales, void *dst, int n_mat,
+                                 int n_out, int n_in, int flags, void *stream) {
+  GPTOSS_REQUIRE(blocks && scales && dst, GPTOSS_ERR_NULL, "pack_mxfp4: null pointer");
+  const int glu = (flags & GPTOSS_PACK_GLU) ? 1 : 0;
+  GPTOSS_REQUIRE(n_mat >= 1 && n_out > 0 && n_in > 0 && n_out % (glu ? 64 : 32) == 0 && n_in % 64 == 0,
+                 GPTOSS_ERR_DIM, "pack_mxfp4: need n_out %% %d == 0 and n_in %% 64 == 0 (n_out=%d n_in=%d)",
+                 glu ? 64 : 32, n_out, n_in);
+  GPTOSS_REQUIRE(aligned(blocks, 4) && aligned(dst, 16), GPTOSS_ERR_ALIGN,
+                 "pack_mxfp4: blocks must be 4-byte and dst 16-byte aligned");
+  size_t threads = (size_t)(n_out / 32) * (n_in / 64) * 64;
+  dim3 grid((unsigned)((threads + 255) / 256), n_mat);
+  pack_mxfp4_kernel<<<grid, 256, 0, (hipStream_t)stream>>>((const unsigned char *)blocks,
+                                                          (const unsigned char *)scales,
+                                                          (unsigned char *)dst, n_out, n_in, glu);
+  GPTOSS_LAUNCH_CHECK("pack_mxfp4_kernel");
   return GPTOSS_OK;
 }

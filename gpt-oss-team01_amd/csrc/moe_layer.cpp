@@ -92,9 +92,9 @@ extern "C" int gptoss_moe_workspace_views(void *workspace, int B, int E, int k, 
   return GPTOSS_OK;
 }
 
-extern "C" int gptoss_moe_forward(const gptoss_moe_weights *w, const void *t, int B, float *out,
-                                  int accumulate, void *workspace, size_t workspace_bytes,
-                                  void *stream) {
+static int moe_forward_impl(const gptoss_moe_weights *w, const void *t, int B, float *out,
+                            int accumulate, void *workspace, size_t workspace_bytes, void *stream,
+                            int mxfp4) {
   int rc = check_moe(w, t, B, out, workspace, workspace_bytes);
   if (rc != GPTOSS_OK) return rc;
   if (B == 0) return GPTOSS_OK;
@@ -115,6 +115,7 @@ extern "C" int gptoss_moe_forward(const gptoss_moe_weights *w, const void *t, in
   g1.row_ids = ws.sorted_pair_ids;
   g1.top_k = k;
   g1.W = (const bf16_t *)w->w1;
+  g1.w_mxfp4 = mxfp4;
   g1.bias = w->b1;
   g1.out = ws.act;
   g1.tiles = ws.tiles;
@@ -128,6 +129,7 @@ extern "C" int gptoss_moe_forward(const gptoss_moe_weights *w, const void *t, in
   GemmParams g2{};
   g2.A = ws.act;
   g2.W = (const bf16_t *)w->w2;
+  g2.w_mxfp4 = mxfp4;
   g2.bias = w->b2;
   g2.out = ws.y2;
   g2.tiles = ws.tiles;
@@ -138,4 +140,16 @@ extern "C" int gptoss_moe_forward(const gptoss_moe_weights *w, const void *t, in
   if (rc != GPTOSS_OK) return rc;
 
   return run_combine(ws.y2, ws.topk_w, ws.inv_perm, out, B, H, k, accumulate, s);
+}
+
+extern "C" int gptoss_moe_forward(const gptoss_moe_weights *w, const void *t, int B, float *out,
+                                  int accumulate, void *workspace, size_t workspace_bytes,
+                                  void *stream) {
+  return moe_forward_impl(w, t, B, out, accumulate, workspace, workspace_bytes, stream, 0);
+}
+
+extern "C" int gptoss_moe_forward_mxfp4(const gptoss_moe_weights *w, const void *t, int B, float *out,
+                                        int accumulate, void *workspace, size_t workspace_bytes,
+                                        void *stream) {
+  return moe_forward_impl(w, t, B, out, accumulate, workspace, workspace_bytes, stream, 1);
 }

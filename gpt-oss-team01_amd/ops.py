@@ -291,3 +291,56 @@ class Engine:
 
     def __del__(self):
         self.close()
+
+
+def pack_mxfp4(blocks: torch.Tensor, scales: torch.Tensor, glu: bool = False) -> torch.Tensor:
+    """blocks uint8 [n_mat, n_out, n_in/2], scales uint8 [n_mat, n_out, n_in/32] -> packed bytes."""
+    _need_gpu()
+    L = _l.load()
+    blocks, scales = blocks.contiguous(), scales.contiguous()
+    n_mat, n_out, half = blocks.shape
+    n_in = half * 2
+    assert tuple(scales.shape) == (n_mat, n_out, n_in // 32)
+    out = torch.empty(L.gptoss_packed_mxfp4_bytes(n_mat, n_out, n_in), dtype=torch.uint8,
+                      device=blocks.device)
+    _l.check(L.gptoss_pack_mxfp4(_ptr(blocks), _ptr(scales), _ptr(out), n_mat, n_out, n_in,
+                                 _l.PACK_GLU if glu else 0, _stream()))
+    return out
+
+
+class MoeLayerMxfp4(MoeLayer):
+    """MoE block whose expert matrices are MXFP4 (e2m1 codes + one e8m0 scale per 32 inputs)."""
+
+    def __init__(self, w_router, b_router, w1_blocks, w1_scales, b1, w2_blocks, w2_scales, b2,
+                 top_k=4, swiglu_limit=7.0, max_tokens=1024):
+        _need_gpu()
+        self.L = _l.load()
+        E, H = w_router.shape
+        I = w2_blocks.shape[2] * 2
+        assert tuple(w1_blocks.shape) == (E, 2 * I, H // 2) and tuple(w2_blocks.shape) == (E, H, I // 2)
+        self.E, self.H, self.I, self.k = E, H, I, top_k
+        dev = w_router.device
+        self.w_router = w_router.to(torch.bfloat16).contiguous()
+        self.b_router = b_router.to(torch.float32).contiguous()
+        self.w1 = pack_mxfp4(w1_blocks, w1_scales, glu=True)
+        self.b1 = b1.to(torch.float32).contiguous()
+        self.w2 = pack_mxfp4(w2_blocks, w2_scales)
+        self.b2 = b2.to(torch.float32).contiguous()
+        self.desc = _l.MoeWeights(E, top_k, H, I, swiglu_limit, self.w_router.data_ptr(),
+                                  self.b_router.data_ptr(), self.w1.data_ptr(),
+                                  self.b1.data_ptr(), self.w2.data_ptr(), self.b2.data_ptr())
+        self.max_tokens = max_tokens
+        self.ws_bytes = self.L.gptoss_moe_workspace_bytes(max_tokens, E, top_k, H, I)
+        self.ws = torch.empty(self.ws_bytes, dtype=torch.uint8, device=dev)
+        self._last_B = 0
+
+    def forward(self, t, out=None, accumulate=False):
+        B = t.shape[0]
+        assert B <= self.max_tokens and t.dtype == torch.bfloat16 and t.is_contiguous()
+        if out is None:
+            out = torch.empty(B, self.H, dtype=torch.float32, device=t.device)
+        _l.check(self.L.gptoss_moe_forward_mxfp4(C.byref(self.desc), _ptr(t), B, _ptr(out),
+                                                 1 if accumulate else 0, _ptr(self.ws),
+                                                 self.ws_bytes, _stream()))
+        self._last_B = B
+        return out

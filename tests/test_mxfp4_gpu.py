@@ -1,0 +1,95 @@
+"""MXFP4 expert weights: the packed FP4 path must reproduce the bf16 path on the dequantised
+weights (the expansion to bf16 is exact, so the two are compared bit for bit), and both must match
+the CPU oracle on the dequantised weights within the bf16 tolerance."""
+import numpy as np
+import pytest
+import torch
+
+from conftest import TOL_MAX, TOL_MEAN, rel_errors
+
+pytestmark = pytest.mark.gpu
+
+
+def _rand_mxfp4(rng, *shape_out_in, exp_lo=-8, exp_hi=0):
+    *lead, n_out, n_in = shape_out_in
+    blocks = rng.integers(0, 256, size=(*lead, n_out, n_in // 2), dtype=np.uint8)
+    scales = (127 + rng.integers(exp_lo, exp_hi + 1, size=(*lead, n_out, n_in // 32))).astype(np.uint8)
+    return blocks, scales
+
+
+def _dequant(orc, blocks, scales):
+    *lead, n_out, half = blocks.shape
+    d = orc.mxfp4_dequant(blocks.reshape(-1, 16), scales.reshape(-1))
+    return d.reshape(*lead, n_out, half * 2)
+
+
+@pytest.mark.parametrize("B,E,H,I,skew", [(64, 8, 256, 256, False), (300, 8, 256, 512, True),
+                                          (200, 128, 2880, 2880, True)])
+def test_mxfp4_matches_bf16_path_and_oracle(ops, orc, B, E, H, I, skew):
+    rng = np.random.default_rng(B + E)
+    w1b, w1s = _rand_mxfp4(rng, E, 2 * I, H)
+    w2b, w2s = _rand_mxfp4(rng, E, H, I)
+    # scale the dequantised magnitudes (|code| <= 6, scale <= 1) down through the activations
+    t = torch.from_numpy(rng.standard_normal((B, H)).astype(np.float32) * 0.05).to(torch.bfloat16)
+    wr = torch.from_numpy(rng.standard_normal((E, H)).astype(np.float32) * 0.02).to(torch.bfloat16)
+    br = np.zeros(E, np.float32)
+    if skew:   # Zipf(1.1) router bias over a fixed permutation of the experts
+        ranks = rng.permutation(E) + 1
+        br = (np.log(1.0 / ranks ** 1.1)).astype(np.float32)
+    br_t = torch.from_numpy(br)
+    b1 = torch.from_numpy(rng.standard_normal((E, 2 * I)).astype(np.float32) * 0.02).to(torch.bfloat16)
+    b2 = torch.from_numpy(rng.standard_normal((E, H)).astype(np.float32) * 0.02).to(torch.bfloat16)
+    w1d, w2d = _dequant(orc, w1b, w1s), _dequant(orc, w2b, w2s)
+    assert np.array_equal(w1d, torch.from_numpy(w1d).to(torch.bfloat16).float().numpy())  # exact in bf16
+
+    fp4 = ops.MoeLayerMxfp4(wr.cuda(), br_t.cuda(), torch.from_numpy(w1b).cuda(), torch.from_numpy(w1s).cuda(),
+                            b1.cuda(), torch.from_numpy(w2b).cuda(), torch.from_numpy(w2s).cuda(), b2.cuda(),
+                            max_tokens=B)
+    ref = ops.MoeLayer(wr.cuda(), br_t.cuda(), torch.from_numpy(w1d).to(torch.bfloat16).cuda(), b1.cuda(),
+                       torch.from_numpy(w2d).to(torch.bfloat16).cuda(), b2.cuda(), max_tokens=B)
+    got = fp4.forward(t.cuda())
+    want_gpu = ref.forward(t.cuda())
+    torch.cuda.synchronize()
+    assert torch.equal(got, want_gpu)                       # same bf16 operands, same MFMA order
+    logits, tw, ti, off, srt, inv = [x.cpu().numpy() for x in fp4.routing_views()]
+    if skew:
+        counts = np.diff(off)
+        assert counts.max() >= 2 * max(1, counts.mean())    # the load really is skewed
+    n_chk = min(B, 48)
+    want, _, _, oti = orc.moe_layer(t.float().numpy()[:n_chk], wr.float().numpy(), br, w1d, b1.float().numpy(),
+                                    w2d, b2.float().numpy(), k=4, limit=7.0, stage=orc.STAGE_SWIGLU,
+                                    want_routing=True)
+    same = (oti == ti[:n_chk]).all(axis=1)
+    assert same.mean() > 0.9
+    mx, mean = rel_errors(got.cpu().numpy()[:n_chk][same], want[same])
+    assert mx <= TOL_MAX and mean <= TOL_MEAN, (mx, mean)
+
+
+def test_mxfp4_every_code_and_scale_expands_exactly(ops, orc):
+    """A one-expert layer with identity-like activations reads back every (code, scale) pair."""
+    E, H, I, B = 1, 64, 64, 64
+    rng = np.random.default_rng(0)
+    # w2 rows enumerate all 16 codes; scales sweep a wide range
+    w2b = np.zeros((E, H, I // 2), np.uint8)
+    for r in range(H):
+        for j in range(I // 2):
+            lo, hi = (r + 2 * j) % 16, (r + 2 * j + 1) % 16
+            w2b[0, r, j] = lo | (hi << 4)
+    w2s = (127 + (np.arange(H)[:, None] % 41 - 20 + np.arange(I // 32)[None, :] * 3)).astype(np.uint8)[None]
+    w1b, w1s = _rand_mxfp4(rng, E, 2 * I, H)
+    fp4_w2 = ops.pack_mxfp4(torch.from_numpy(w2b).cuda(), torch.from_numpy(w2s).cuda())
+    w2d = _dequant(orc, w2b, w2s)
+    bf_w2 = ops.pack_weight(torch.from_numpy(w2d).to(torch.bfloat16).cuda())
+    # run GEMM2 alone through the layer by comparing full layers that differ only in w2's format
+    wr = torch.zeros(E, H, dtype=torch.bfloat16)
+    z1 = torch.zeros(E, 2 * I)
+    z2 = torch.zeros(E, H)
+    t = torch.from_numpy(rng.standard_normal((B, H)).astype(np.float32)).to(torch.bfloat16)
+    a = ops.MoeLayerMxfp4(wr.cuda(), torch.zeros(E).cuda(), torch.from_numpy(w1b).cuda(), torch.from_numpy(w1s).cuda(),
+                          z1.cuda(), torch.from_numpy(w2b).cuda(), torch.from_numpy(w2s).cuda(), z2.cuda(),
+                          top_k=1, max_tokens=B)
+    w1d = _dequant(orc, w1b, w1s)
+    b = ops.MoeLayer(wr.cuda(), torch.zeros(E).cuda(), torch.from_numpy(w1d).to(torch.bfloat16).cuda(), z1.cuda(),
+                     torch.from_numpy(w2d).to(torch.bfloat16).cuda(), z2.cuda(), top_k=1, max_tokens=B)
+    assert torch.equal(a.forward(t.cuda()), b.forward(t.cuda()))
+    assert fp4_w2.numel() == H * I // 2 + H * I // 32 and bf_w2.numel() == H * I
