@@ -80,11 +80,11 @@ int gptoss_pack_weight(const void *src, void *dst, int n_mat, int n_out, int n_i
 /* logits[B,E] = t[B,H] . w_router[E,H]^T + b_router[E]     (bf16 x bf16 -> fp32)
  * Replaces router_gemm_batched_quantize (getp-csrc/src/layer_hip_batch.cpp:1006-1044).
  * t bf16 [B,H]; w_router bf16 [E,H] row-major (unpacked); b_router fp32 [E] or NULL.
- * Needs H % 32 == 0, E % 16 == 0, E <= 256. */
+ * Needs H % 32 == 0 and 1 <= E <= 256. */
 int gptoss_router_gemm(const void *t, const void *w_router, const float *b_router, float *logits,
                        int B, int H, int E, void *stream);
 
-/* Sizes of the routing outputs for B tokens: ints in the tile list. */
+/* Upper bound of the number of (expert,row0,rows) entries gptoss_moe_route can write for B tokens. */
 int gptoss_moe_max_tiles(int B, int k, int E, int rows_per_tile);
 
 /* Top-k gating and expert grouping from router logits.  Replaces
@@ -99,7 +99,7 @@ int gptoss_moe_max_tiles(int B, int k, int E, int rows_per_tile);
  * sorted_pair_ids int32 [B*k], inv_perm int32 [B*k] (inv_perm[pair] = its row in the sorted
  * order), tiles int32 [1 + 3*gptoss_moe_max_tiles()] = {n_tiles, (expert,row0,rows)...} cutting
  * every expert's rows into tiles of rows_per_tile (may be NULL with rows_per_tile 0).
- * Needs 1 <= k <= 8, k <= E, E % 32 == 0, E <= 256, rows_per_tile in {0,32,64,128,256}. */
+ * Needs 1 <= k <= 8, k <= E <= 256, rows_per_tile in {0,32,64,128,256}. */
 int gptoss_moe_route(const float *logits, int B, int E, int k, float *topk_w, int *topk_i,
                      int *expert_offsets, int *sorted_pair_ids, int *inv_perm, int *tiles,
                      int rows_per_tile, void *stream);
@@ -130,7 +130,8 @@ size_t gptoss_moe_workspace_bytes(int B, int E, int k, int H, int I);
  * with the token gather folded into its operand load and clamped SwiGLU folded into its epilogue
  * (kernel.cpp:560-573,636-685,927-952), grouped GEMM2 (kernel.cpp:1061-1089) and a deterministic
  * per-token weighted combine in slot order (replaces the atomicAdd scatter, kernel.cpp:748-768).
- * t bf16 [B,H]; out fp32 [B,H].  Needs H % 64 == 0, I % 64 == 0, E % 32 == 0, E <= 256, k <= 8. */
+ * t bf16 [B,H]; out fp32 [B,H].  Needs H % 64 == 0, I % 64 == 0, k <= min(8,E), E <= 256,
+ * B*k*max(H,I) < 2^31. */
 int gptoss_moe_forward(const gptoss_moe_weights *w, const void *t, int B, float *out,
                        int accumulate, void *workspace, size_t workspace_bytes, void *stream);
 
@@ -198,8 +199,8 @@ typedef struct gptoss_engine gptoss_engine;
 
 enum {
   GPTOSS_ENGINE_SYNTHETIC = 1, /* host_weights ignored: N(0,0.02) bf16 weights generated on device */
-  GPTOSS_ENGINE_PRECISE = 2    /* keep activations at fp32 accuracy in every GEMM (3-term bf16
-                                  split) instead of the reference GPU path's bf16 staging */
+  GPTOSS_ENGINE_PRECISE = 2    /* reserved: fp32-faithful activations instead of the reference GPU
+                                  path's bf16 staging; engine_create refuses it in this version */
 };
 
 /* Build device weights (bf16, packed) and run state for up to max_batch sequences of up to
