@@ -190,8 +190,14 @@ int dense_gemm(const bf16_t *A, const bf16_t *W, const float *bias, void *out, i
   g.n_col_tiles = cdiv(N, 256);
   // largest row tile that still gives the 256 CUs at least one workgroup each; the weights of
   // these GEMMs are small enough to be re-read from L2 by the extra row tiles
-  int rpt = 256;
-  while (rpt > 32 && (rpt / 2 >= B || cdiv(B, rpt) * g.n_col_tiles < 256)) rpt /= 2;
+  static const int sizes[4] = {160, 128, 64, 32};
+  int rpt = 32;
+  for (int i = 0; i < 4; i++) {
+    rpt = sizes[i];
+    if (rpt == 32) break;
+    if (sizes[i + 1] >= B) continue;  // a smaller tile still holds every row
+    if (cdiv(B, rpt) * g.n_col_tiles >= 256) break;
+  }
   return run_gemm(g, false, epi, rpt, cdiv(B, rpt), s);
 }
 

@@ -27,5 +27,10 @@ int run_gemm(const GemmParams &p, bool gather, int epi, int rows_per_tile, int m
 int run_combine(const float *y2, const float *topk_w, const int *inv_perm, float *out, int B, int H,
                 int k, int accumulate, hipStream_t s);
 int moe_rows_per_tile(int B, int k, int E);
+// moe_route.hip
+int run_router(const void *t, const void *w_router, const float *b_router, float *logits, int B,
+               int H, int E, int k, float *topk_w, int *topk_i, hipStream_t s);
+int run_group(int B, int E, int k, float *topk_w, int *topk_i, int *expert_offsets,
+              int *sorted_pair_ids, int *inv_perm, int *tiles, int rows_per_tile, hipStream_t s);
 
 }  // namespace gptoss

@@ -1,0 +1,453 @@
+// Grouped (per-expert) and dense bf16 GEMMs for gfx950 built on v_mfma_f32_32x32x16_bf16.
+//
+//   C[rows, N] = A[rows, K] . W[N, K]^T      rows = the tokens routed to one expert (or a slice
+//                                            of a dense batch), W = that expert's matrix
+//
+// Shape of the problem at decode time: a few hundred rows per expert against 25 M weights per
+// expert, i.e. every weight is used by ~128 rows and the kernel is bound by streaming W from
+// HBM.  The design follows from that:
+//   * W is stored in MFMA-fragment order (gptoss_pack_weight): the 1 KB a wave needs for one
+//     32-column x 16-k operand is contiguous, so each wave streams its own columns with
+//     perfectly coalesced 128-bit loads straight into registers (no LDS hop, no reuse needed:
+//     a workgroup covers all rows of its tile, up to 160, so W is read once);
+//   * the activations (shared by the 4 waves) go through a double-buffered, padded LDS tile; the
+//     token gather of the reference's pack step is folded into that load;
+//   * a workgroup = 256 virtual columns x up to 160 rows; each wave owns 64 columns as two
+//     B fragments and reuses every A fragment it reads from LDS for two MFMAs;
+//   * work items come from the device-built tile list (expert,row0,rows), mapped so that the
+//     workgroups of one XCD walk consecutive column tiles of the same expert (A stays in that
+//     XCD's L2);
+//   * epilogues: +bias -> fp32, or +bias -> clamped SwiGLU -> bf16 with gate and up of a pair in
+//     the same lane (arranged by the packing order, so no cross-lane traffic).
+#pragma once
+
+#include <type_traits>
+
+#include "common.hpp"
+#include "gemm.hpp"
+
+namespace gptoss {
+
+constexpr int GEMM_THREADS = 256;
+constexpr int BK = 64;            // k per LDS slab (4 MFMA k-steps)
+constexpr int LDS_ROW = BK + 8;   // padded row length in bf16 elements (144 B)
+constexpr int BN = 256;           // virtual columns per workgroup (4 waves x 64)
+
+// MXFP4 operand expansion.  One dword holds the lane's 8 e2m1 codes of a k-step (element j < 4 in
+// the low nibble of byte j, element j >= 4 in the high nibble of byte j-4).  tab[] holds the eight
+// positive bf16 magnitudes already multiplied by the block's power-of-two scale, as byte tables
+// for v_perm_b32: tab[0]/tab[1] = low bytes of entries 0-3 / 4-7, tab[2]/tab[3] = high bytes.
+struct Fp4Table {
+  uint32_t lo_a, lo_b, hi_a, hi_b;
+};
+
+__device__ __forceinline__ Fp4Table fp4_table(uint32_t e8m0) {
+  // bf16 bit patterns of 0, .5 | 1, 1.5 | 2, 3 | 4, 6 as pairs; the exponent field starts at bit 7
+  // d * 0x00800080 adds d to both exponent fields: for negative d the borrow out of the low half
+  // is undone by the carry of the low-half addition below
+  const uint32_t dd = (e8m0 - 127u) * 0x00800080u;
+  const uint32_t t01 = 0x3F000000u + ((e8m0 - 127u) << 23);  // entry 0 stays +0
+  const uint32_t t23 = 0x3FC03F80u + dd;
+  const uint32_t t45 = 0x40404000u + dd;
+  const uint32_t t67 = 0x40C04080u + dd;
+  Fp4Table t;
+  // v_perm_b32(S0, S1, sel): selector values 0-3 pick bytes of S1, 4-7 bytes of S0
+  t.lo_a = __builtin_amdgcn_perm(t23, t01, 0x06040200u);
+  t.hi_a = __builtin_amdgcn_perm(t23, t01, 0x07050301u);
+  t.lo_b = __builtin_amdgcn_perm(t67, t45, 0x06040200u);
+  t.hi_b = __builtin_amdgcn_perm(t67, t45, 0x07050301u);
+  return t;
+}
+
+__device__ __forceinline__ u32x4 fp4_expand(uint32_t w, const Fp4Table &t) {
+  const uint32_t m_lo = w & 0x07070707u, m_hi = (w >> 4) & 0x07070707u;
+  uint32_t l0 = __builtin_amdgcn_perm(t.lo_b, t.lo_a, m_lo);
+  uint32_t h0 = __builtin_amdgcn_perm(t.hi_b, t.hi_a, m_lo) | ((w << 4) & 0x80808080u);
+  uint32_t l1 = __builtin_amdgcn_perm(t.lo_b, t.lo_a, m_hi);
+  uint32_t h1 = __builtin_amdgcn_perm(t.hi_b, t.hi_a, m_hi) | (w & 0x80808080u);
+  // interleave low and high bytes into bf16 pairs: elements 0,1 | 2,3 | 4,5 | 6,7
+  return u32x4{__builtin_amdgcn_perm(h0, l0, 0x05010400u), __builtin_amdgcn_perm(h0, l0, 0x07030602u),
+               __builtin_amdgcn_perm(h1, l1, 0x05010400u), __builtin_amdgcn_perm(h1, l1, 0x07030602u)};
+}
+
+template <int I, int N, typename F>
+__device__ __forceinline__ void static_for(F &&f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>{});
+    static_for<I + 1, N>(f);
+  }
+}
+
+// Where one wave's two W fragment streams of a work item start.
+struct WStream {
+  const bf16_t *w;           // bf16: first fragment of the wave's first 32-column block
+  const unsigned char *c;    // MXFP4: codes
+  const unsigned char *sc;   // MXFP4: scales
+};
+
+template <bool FP4>
+__device__ __forceinline__ WStream w_stream(const GemmParams &p, int mat, int ct, int wave) {
+  const int K = p.K, N = p.N;
+  int n0 = ct * BN + wave * 64;
+  if (n0 >= N) n0 = N - 64;  // idle waves of the last column tile stream a valid block again
+  WStream st{nullptr, nullptr, nullptr};
+  if (FP4) {
+    const int nslab = K / BK;
+    const size_t mat_bytes = (size_t)N * K / 2 + (size_t)N * K / 32;
+    const unsigned char *mb_ = reinterpret_cast<const unsigned char *>(p.W) + (size_t)mat * mat_bytes;
+    st.c = mb_ + (size_t)(n0 >> 5) * nslab * 1024;
+    st.sc = mb_ + (size_t)N * K / 2 + (size_t)(n0 >> 5) * nslab * 64;
+  } else {
+    st.w = p.W + (size_t)mat * N * K + (size_t)(n0 >> 5) * (K / 16) * 512;
+  }
+  return st;  // wave-uniform; each lane adds its own 16 bytes (2 scale bytes) when loading
+}
+
+// Register ring holding NRING slabs of the wave's W operands.
+template <int NRING, bool FP4>
+struct WRing {
+  static constexpr int BQ = FP4 ? 1 : 4;
+  u32x4 b[NRING][2][BQ];
+  uint32_t s[NRING][2];
+};
+
+template <int NRING, bool FP4, int R>
+__device__ __forceinline__ void w_load(WRing<NRING, FP4> &ring, const WStream &st, int slab, int K,
+                                       int lane, std::integral_constant<int, R>) {
+  if (FP4) {
+    const int nslab = K / BK;
+#pragma unroll
+    for (int f = 0; f < 2; f++) {
+      ring.b[R][f][0] = *reinterpret_cast<const u32x4 *>(st.c + (size_t)f * nslab * 1024 +
+                                                         (size_t)slab * 1024 + lane * 16);
+      ring.s[R][f] = *reinterpret_cast<const unsigned short *>(st.sc + (size_t)f * nslab * 64 +
+                                                               (size_t)slab * 64 + (lane & 31) * 2);
+    }
+  } else {
+    const size_t frag_stride = (size_t)(K / 16) * 512;  // elements between adjacent 32-column blocks
+#pragma unroll
+    for (int f = 0; f < 2; f++)
+#pragma unroll
+      for (int kk = 0; kk < 4; kk++)
+        ring.b[R][f][kk % WRing<NRING, FP4>::BQ] =
+            *reinterpret_cast<const u32x4 *>(st.w + f * frag_stride + (size_t)(slab * 4 + kk) * 512 + lane * 8);
+  }
+}
+
+// One (row tile, column tile) work item with a compile-time number of 32-row blocks, so every
+// loop below is fully unrolled and every global load is unconditional.  On entry the ring holds
+// slabs 0..NRING-2 of this item's W streams; while the last slabs are multiplied the ring is
+// refilled from `next` (the streams of the workgroup's next work item), so the HBM stream of W
+// never drains between work items.  On exit the ring holds slabs 0..NRING-2 of `next`.
+template <int MB, int NRING, bool GATHER, int EPI, bool FP4>
+__device__ __forceinline__ void gemm_tile(const GemmParams &p, bf16_t *lds, int lds_stage, int mat,
+                                          int row0, int rows, int ct, WRing<NRING, FP4> &ring,
+                                          const WStream &cur, const WStream &next) {
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int K = p.K, N = p.N;
+  const int n0_raw = ct * BN + wave * 64;
+  const bool wave_active = n0_raw < N;
+  const int n0 = wave_active ? n0_raw : N - 64;
+  const int nslab = K / BK;
+  constexpr int D = NRING - 1;  // slabs of W in flight
+  constexpr int BQ = WRing<NRING, FP4>::BQ;
+
+  // ---- A: each thread moves one 16-byte chunk per 32-row block and slab -----------------------
+  const int a_row = tid >> 3, a_kc = tid & 7;
+  uint32_t a_off[MB];
+#pragma unroll
+  for (int i = 0; i < MB; i++) {
+    int r = a_row + 32 * i;
+    int src = GATHER ? 0 : row0;
+    if (r < rows) {
+      if (GATHER) src = p.row_ids[row0 + r] / p.top_k;
+      else src = row0 + r;
+    }
+    a_off[i] = (uint32_t)src * (uint32_t)K + a_kc * 8;
+  }
+  u32x4 areg[MB];
+  auto load_a = [&](int s) {
+#pragma unroll
+    for (int i = 0; i < MB; i++) areg[i] = *reinterpret_cast<const u32x4 *>(p.A + a_off[i] + s * BK);
+  };
+  bf16_t *a_dst = lds + a_row * LDS_ROW + a_kc * 8;
+  auto store_a = [&](int stage) {
+#pragma unroll
+    for (int i = 0; i < MB; i++)
+      *reinterpret_cast<u32x4 *>(a_dst + stage * lds_stage + 32 * i * LDS_ROW) = areg[i];
+  };
+
+  auto zero_a = [&](int stage) {
+#pragma unroll
+    for (int i = 0; i < MB; i++)
+      *reinterpret_cast<u32x4 *>(a_dst + stage * lds_stage + 32 * i * LDS_ROW) = u32x4{0u, 0u, 0u, 0u};
+  };
+
+  f32x16 acc[MB][2];
+#pragma unroll
+  for (int i = 0; i < MB; i++)
+#pragma unroll
+    for (int f = 0; f < 2; f++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[i][f][r] = 0.f;
+
+  const bf16_t *a_src = lds + (lane & 31) * LDS_ROW + (lane >> 5) * 8;
+  bf16x8 af[2][MB];
+  auto compute = [&](int stage, auto rsel) {
+    constexpr int R = decltype(rsel)::value;
+    const bf16_t *base = a_src + stage * lds_stage;
+    Fp4Table tab[2][2];
+    if (FP4) {
+#pragma unroll
+      for (int f = 0; f < 2; f++) {
+        tab[f][0] = fp4_table(ring.s[R][f] & 0xffu);
+        tab[f][1] = fp4_table((ring.s[R][f] >> 8) & 0xffu);
+      }
+    }
+    // af[0] already holds the fragments of k-step 0 (requested before the previous barrier).  The
+    // fragments of k-step kk+1 are requested before the MFMAs of k-step kk are issued, and the
+    // scheduling fences keep the compiler from sinking those reads next to their uses.
+#pragma unroll
+    for (int kk = 0; kk < 4; kk++) {
+      if (kk + 1 < 4) {
+#pragma unroll
+        for (int i = 0; i < MB; i++)
+          af[(kk + 1) & 1][i] =
+              as_bf16x8(*reinterpret_cast<const u32x4 *>(base + i * 32 * LDS_ROW + (kk + 1) * 16));
+      }
+      bf16x8 b0, b1;
+      if (FP4) {
+        b0 = as_bf16x8(fp4_expand(ring.b[R][0][0][kk], tab[0][kk >> 1]));
+        b1 = as_bf16x8(fp4_expand(ring.b[R][1][0][kk], tab[1][kk >> 1]));
+      } else {
+        b0 = as_bf16x8(ring.b[R][0][kk % BQ]);
+        b1 = as_bf16x8(ring.b[R][1][kk % BQ]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < MB; i++) {
+        acc[i][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[kk & 1][i], b0, acc[i][0], 0, 0, 0);
+        acc[i][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[kk & 1][i], b1, acc[i][1], 0, 0, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  auto read_first_frags = [&](int stage) {
+    const bf16_t *base = a_src + stage * lds_stage;
+#pragma unroll
+    for (int i = 0; i < MB; i++)
+      af[0][i] = as_bf16x8(*reinterpret_cast<const u32x4 *>(base + i * 32 * LDS_ROW));
+  };
+
+  // Three LDS stages for A: slab s is multiplied from stage s%3 while slab s+2 is being written
+  // to stage (s+2)%3, so the first fragments of slab s+1 (complete since the previous barrier) can
+  // be requested before this iteration's barrier and their latency is hidden behind it.
+  // The slab loop runs a multiple of NRING iterations so the ring is back at index 0 for the next
+  // item; the (at most NRING-1) padding iterations multiply zero A rows.
+  const int last = nslab - 1;
+  const int padded = (nslab + NRING - 1) / NRING * NRING;
+  load_a(0);
+  store_a(0);
+  if (nslab > 1) {
+    load_a(1);
+    store_a(1);
+  } else {
+    zero_a(1);
+  }
+  load_a(min(2, last));
+  __syncthreads();
+  read_first_frags(0);
+
+  int st = 0;  // s % 3
+  auto body = [&](int s, auto rsel) {
+    constexpr int R = decltype(rsel)::value;
+    using Refill = std::integral_constant<int, (R + D) % NRING>;
+    // ring slot consumed at iteration s+D: slab s+D of this item, nothing useful while padding,
+    // then the first slabs of the next item
+    const int t = s + D;
+    const bool wrap = t >= padded;
+    w_load<NRING, FP4>(ring, wrap ? next : cur, wrap ? t - padded : min(t, last), K, lane, Refill{});
+    compute(st, rsel);
+    const int st1 = (st == 2) ? 0 : st + 1, st2 = (st1 == 2) ? 0 : st1 + 1;
+    if (s + 2 < nslab) store_a(st2);  // rows of slab s+2
+    else zero_a(st2);
+    load_a(min(s + 3, last));
+    read_first_frags(st1);
+    st = st1;
+    __syncthreads();
+  };
+  for (int s = 0; s < padded; s += NRING)
+    static_for<0, NRING>([&](auto r) { body(s + (int)decltype(r)::value, r); });
+
+  if (!wave_active) return;
+
+  // ---- epilogue ------------------------------------------------------------------------------
+  const int c = lane & 31, rsub = (lane >> 5) * 4;
+  if (EPI == EPI_SWIGLU) {
+    const int half_n = N >> 1;
+    const int j = (n0 >> 1) + c;  // pair index: gate = row 2j, up = row 2j+1 of the .bin matrix
+    float bg = 0.f, bu = 0.f;
+    if (p.bias) {
+      bg = p.bias[(size_t)mat * N + 2 * j];
+      bu = p.bias[(size_t)mat * N + 2 * j + 1];
+    }
+    bf16_t *o = reinterpret_cast<bf16_t *>(p.out);
+    const float L = p.limit;
+#pragma unroll
+    for (int i = 0; i < MB; i++) {
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        int row = i * 32 + (r >> 2) * 8 + rsub + (r & 3);
+        if (row < rows) {
+          float g = acc[i][0][r] + bg, u = acc[i][1][r] + bu;
+          g = fminf(g, L);
+          u = fminf(fmaxf(u, -L), L);
+          float v = g * (1.0f / (1.0f + expf(-1.702f * g)));
+          v *= (u + 1.0f);
+          o[(size_t)(row0 + row) * half_n + j] = f32_to_bf16(v);
+        }
+      }
+    }
+  } else {
+#pragma unroll
+    for (int f = 0; f < 2; f++) {
+      const int col = n0 + f * 32 + c;
+      float bv = p.bias ? p.bias[(size_t)mat * N + col] : 0.f;
+#pragma unroll
+      for (int i = 0; i < MB; i++) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          int row = i * 32 + (r >> 2) * 8 + rsub + (r & 3);
+          if (row < rows) {
+            float v = acc[i][f][r] + bv;
+            if (EPI == EPI_F32)
+              reinterpret_cast<float *>(p.out)[(size_t)(row0 + row) * N + col] = v;
+            else
+              reinterpret_cast<bf16_t *>(p.out)[(size_t)(row0 + row) * N + col] = f32_to_bf16(v);
+          }
+        }
+      }
+    }
+  }
+}
+
+// NRING: slabs of W held in registers per wave, NRING-1 of them in flight.
+template <int MBMAX>
+struct RingDepth {
+  static constexpr int value = 3;
+};
+
+// Persistent kernel: the grid is one workgroup per CU (two for the small-tile kernels); workgroups
+// are dealt round-robin to the 8 XCDs, XCD x owns the x-th contiguous eighth of the work list
+// (consecutive column tiles of the same expert, so that expert's rows stay in that XCD's L2) and
+// its workgroups walk that eighth with a stride of the number of workgroups per XCD.
+template <int MBMAX, bool GATHER, int EPI, bool FP4>
+__global__ __launch_bounds__(GEMM_THREADS) void grouped_gemm_kernel(GemmParams p) {
+  constexpr int BM = MBMAX * 32;
+  constexpr int NRING = RingDepth<MBMAX>::value;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  bf16_t *lds = reinterpret_cast<bf16_t *>(smem_raw);  // [3][BM][LDS_ROW]
+  constexpr int STAGE = BM * LDS_ROW;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+
+  const int n_tiles = p.tiles ? p.tiles[0] : (p.dense_rows + BM - 1) / BM;
+  const int total = n_tiles * p.n_col_tiles;
+  const int chunk = (total + 7) >> 3;
+  const int per_xcd = gridDim.x >> 3;
+  const int xcd = blockIdx.x & 7;
+  int j = blockIdx.x >> 3;
+  auto valid = [&](int jj) { return jj < chunk && xcd * chunk + jj < total; };
+  if (!valid(j)) return;
+
+  struct Item {
+    int mat, row0, rows, ct;
+  };
+  auto decode = [&](int jj) {
+    const int work = xcd * chunk + jj;
+    const int tile = work / p.n_col_tiles;
+    Item it;
+    it.ct = work - tile * p.n_col_tiles;
+    if (p.tiles) {
+      it.mat = p.tiles[1 + 3 * tile];
+      it.row0 = p.tiles[2 + 3 * tile];
+      it.rows = p.tiles[3 + 3 * tile];
+    } else {
+      it.mat = 0;
+      it.row0 = tile * BM;
+      it.rows = min(BM, p.dense_rows - it.row0);
+    }
+    return it;
+  };
+
+  Item cur = decode(j);
+  WStream cur_w = w_stream<FP4>(p, cur.mat, cur.ct, wave);
+  WRing<NRING, FP4> ring;
+  static_for<0, NRING - 1>([&](auto r) {
+    w_load<NRING, FP4>(ring, cur_w, min((int)decltype(r)::value, p.K / BK - 1), p.K, lane, r);
+  });
+  while (true) {
+    const int jn = j + per_xcd;
+    const bool more = valid(jn);
+    const Item nxt = more ? decode(jn) : cur;
+    // without a next item the refill re-reads this item's first slabs: harmless and unconditional
+    const WStream nxt_w = more ? w_stream<FP4>(p, nxt.mat, nxt.ct, wave) : cur_w;
+    // one fully unrolled code path per number of 32-row blocks actually present in the tile
+    const int mb = (cur.rows + 31) >> 5;
+    bool done = false;
+    static_for<1, MBMAX + 1>([&](auto m) {
+      constexpr int M = decltype(m)::value;
+      if (!done && (mb == M || M == MBMAX)) {
+        gemm_tile<M, NRING, GATHER, EPI, FP4>(p, lds, STAGE, cur.mat, cur.row0, cur.rows, cur.ct, ring,
+                                              cur_w, nxt_w);
+        done = true;
+      }
+    });
+    if (!more) break;
+    // every wave must be done reading this item's last A slab before the next prologue overwrites it
+    __syncthreads();
+    j = jn;
+    cur = nxt;
+    cur_w = nxt_w;
+  }
+}
+
+template <int MBMAX, bool GATHER, int EPI, bool FP4>
+int launch_gemm(const GemmParams &p, int max_tiles, hipStream_t s) {
+  static bool attr_done = false;
+  size_t smem = (size_t)3 * MBMAX * 32 * LDS_ROW * sizeof(bf16_t);
+  auto kern = grouped_gemm_kernel<MBMAX, GATHER, EPI, FP4>;
+  if (!attr_done) {
+    GPTOSS_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+    attr_done = true;
+  }
+  int total = max_tiles * p.n_col_tiles;
+  // one resident workgroup per CU for the large tiles (their registers allow no more), two for
+  // the small ones
+  const int resident = (MBMAX <= 2 ? 2 : 1) * 256;
+  int grid = ((total + 7) / 8) * 8;
+  if (grid > resident) grid = resident;
+  if (grid == 0) return GPTOSS_OK;
+  {
+    TraceScope ts(FP4 ? (GATHER ? "gemm1_gather_swiglu_mxfp4" : "gemm_f32_mxfp4")
+                      : (GATHER ? "gemm1_gather_swiglu" : "gemm_f32"), s);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(GEMM_THREADS), smem, s, p);
+  }
+  GPTOSS_LAUNCH_CHECK("grouped_gemm_kernel");
+  return GPTOSS_OK;
+}
+
+// the two operand/epilogue combinations in use, for every row-tile size
+#define GPTOSS_GEMM_INSTANTIATE(FP4V)                                                          \
+  template int launch_gemm<1, true, EPI_SWIGLU, FP4V>(const GemmParams &, int, hipStream_t);   \
+  template int launch_gemm<2, true, EPI_SWIGLU, FP4V>(const GemmParams &, int, hipStream_t);   \
+  template int launch_gemm<4, true, EPI_SWIGLU, FP4V>(const GemmParams &, int, hipStream_t);   \
+  template int launch_gemm<5, true, EPI_SWIGLU, FP4V>(const GemmParams &, int, hipStream_t);   \
+  template int launch_gemm<1, false, EPI_F32, FP4V>(const GemmParams &, int, hipStream_t);     \
+  template int launch_gemm<2, false, EPI_F32, FP4V>(const GemmParams &, int, hipStream_t);     \
+  template int launch_gemm<4, false, EPI_F32, FP4V>(const GemmParams &, int, hipStream_t);     \
+  template int launch_gemm<5, false, EPI_F32, FP4V>(const GemmParams &, int, hipStream_t);
+
+}  // namespace gptoss

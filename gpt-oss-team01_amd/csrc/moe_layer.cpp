@@ -1,6 +1,8 @@
 // Host side of the MoE block: workspace layout and the launch sequence
 // router GEMM -> top-k/softmax -> stable grouping + tile list -> grouped GEMM1 (+gather, +SwiGLU)
 // -> grouped GEMM2 -> ordered weighted combine.  Nothing here synchronises or allocates.
+#include <math.h>
+
 #include "common.hpp"
 #include "gemm.hpp"
 
@@ -36,12 +38,16 @@ static MoeWorkspace carve(void *base, int B, int E, int k, int H, int I) {
   return w;
 }
 
+// Row-tile size (32, 64, 128 or 160 rows) for B*k pairs over E experts: the smallest tile that holds an average
+// expert's rows plus 2.5 standard deviations of a uniform routing, so that nearly every expert is
+// a single tile (its weights are then streamed exactly once).
 int moe_rows_per_tile(int B, int k, int E) {
-  long long avg = ((long long)B * k + E - 1) / E;
-  if (avg <= 21) return 32;
-  if (avg <= 42) return 64;
-  if (avg <= 85) return 128;
-  return 256;
+  double avg = (double)B * k / E;
+  double need = avg + 2.5 * sqrt(avg);
+  if (need <= 32) return 32;
+  if (need <= 64) return 64;
+  if (need <= 128) return 128;
+  return 160;
 }
 
 static int check_moe(const gptoss_moe_weights *w, const void *t, int B, float *out, void *ws,
@@ -51,6 +57,7 @@ static int check_moe(const gptoss_moe_weights *w, const void *t, int B, float *o
   const int E = w->n_experts, k = w->top_k, H = w->hidden, I = w->intermediate;
   GPTOSS_REQUIRE(B >= 0 && E >= 1 && E <= 256 && k >= 1 && k <= 8 && k <= E, GPTOSS_ERR_DIM,
                  "moe_forward: need 1 <= k <= min(8,E), E <= 256 (B=%d E=%d k=%d)", B, E, k);
+  GPTOSS_REQUIRE(aligned(t, 16), GPTOSS_ERR_ALIGN, "moe_forward: t must be 16-byte aligned");
   GPTOSS_REQUIRE(H > 0 && I > 0 && H % 64 == 0 && I % 64 == 0, GPTOSS_ERR_DIM,
                  "moe_forward: need hidden %% 64 == 0 and intermediate %% 64 == 0 (H=%d I=%d)", H, I);
   GPTOSS_REQUIRE((long long)B * k * (long long)(H > I ? H : I) < (1ll << 31), GPTOSS_ERR_DIM,
@@ -104,10 +111,11 @@ static int moe_forward_impl(const gptoss_moe_weights *w, const void *t, int B, f
   const int rpt = moe_rows_per_tile(B, k, E);
   const int max_tiles = gptoss_moe_max_tiles(B, k, E, rpt);
 
-  rc = gptoss_router_gemm(t, w->w_router, w->b_router, ws.logits, B, H, E, stream);
+  // router GEMM with the gating of its own 16 tokens fused in, then the stable grouping
+  rc = run_router(t, w->w_router, w->b_router, ws.logits, B, H, E, k, ws.topk_w, ws.topk_i, s);
   if (rc != GPTOSS_OK) return rc;
-  rc = gptoss_moe_route(ws.logits, B, E, k, ws.topk_w, ws.topk_i, ws.expert_offsets,
-                        ws.sorted_pair_ids, ws.inv_perm, ws.tiles, rpt, stream);
+  rc = run_group(B, E, k, ws.topk_w, ws.topk_i, ws.expert_offsets, ws.sorted_pair_ids, ws.inv_perm,
+                 ws.tiles, rpt, s);
   if (rc != GPTOSS_OK) return rc;
 
   GemmParams g1{};

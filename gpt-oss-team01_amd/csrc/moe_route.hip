@@ -3,82 +3,20 @@
 // ballots and an LDS histogram (no global atomics), which also emits the tile list that the
 // grouped GEMMs schedule from.
 #include "common.hpp"
+#include "gemm.hpp"
 
 namespace gptoss {
 
 // ------------------------------------------------------------------------------------------------
-// Router GEMM: logits[B,E] = t[B,H] . Wr[E,H]^T + br.  One workgroup = 16 token rows x all experts;
-// its 4 waves split the K loop (k-steps of 32 interleaved) and reduce through LDS.
-// ------------------------------------------------------------------------------------------------
-template <int NB>  // number of 16-expert column blocks held per wave
-__global__ __launch_bounds__(256) void router_gemm_kernel(const bf16_t *__restrict__ t,
-                                                          const bf16_t *__restrict__ wr,
-                                                          const float *__restrict__ br,
-                                                          float *__restrict__ logits, int B, int H,
-                                                          int E) {
-  __shared__ float red[3][16][NB * 16 + 1];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int r0 = blockIdx.x * 16;
-  const int arow = min(r0 + (lane & 15), B - 1);
-  const int kq = (lane >> 4) * 8;
-  const bf16_t *ap = t + (size_t)arow * H + kq;
-  f32x4 acc[NB];
-#pragma unroll
-  for (int nb = 0; nb < NB; nb++) acc[nb] = f32x4{0.f, 0.f, 0.f, 0.f};
-  const int ksteps = H / 32;
-  for (int ks = wave; ks < ksteps; ks += 4) {
-    u32x4 a = *reinterpret_cast<const u32x4 *>(ap + ks * 32);
-#pragma unroll
-    for (int nb = 0; nb < NB; nb++) {
-      int e = nb * 16 + (lane & 15);
-      u32x4 b = u32x4{0u, 0u, 0u, 0u};
-      if (e < E) b = *reinterpret_cast<const u32x4 *>(wr + (size_t)e * H + ks * 32 + kq);
-      acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a), as_bf16x8(b), acc[nb], 0, 0, 0);
-    }
-  }
-  if (wave > 0) {
-#pragma unroll
-    for (int nb = 0; nb < NB; nb++)
-#pragma unroll
-      for (int i = 0; i < 4; i++)
-        red[wave - 1][(lane >> 4) * 4 + i][nb * 16 + (lane & 15)] = acc[nb][i];
-  }
-  __syncthreads();
-  if (wave == 0) {
-#pragma unroll
-    for (int nb = 0; nb < NB; nb++) {
-      int e = nb * 16 + (lane & 15);
-#pragma unroll
-      for (int i = 0; i < 4; i++) {
-        int r = (lane >> 4) * 4 + i;
-        if (e < E && r0 + r < B) {
-          float v = acc[nb][i] + red[0][r][e] + red[1][r][e] + red[2][r][e];
-          if (br) v += br[e];
-          logits[(size_t)(r0 + r) * E + e] = v;
-        }
-      }
-    }
-  }
-}
-
-// ------------------------------------------------------------------------------------------------
-// Top-k + softmax.  32 lanes per token (two tokens per wave); lane j holds experts j, j+32, ...
-// Selection = k rounds of (local best, 5-step butterfly) ordered by (value desc, expert id asc).
+// Top-k + softmax for one token held by a group of 32 lanes: lane j holds experts j, j+32, ...
+// Selection = k rounds of (local best, 5-step butterfly) ordered by (value desc, expert id asc);
+// softmax over the k picked values with exp in float and the sum and division in double
+// (run.cpp:319-337).  Every lane of the group must call; lane 0 of the group writes.
 // ------------------------------------------------------------------------------------------------
 template <int NJ>
-__global__ __launch_bounds__(256) void topk_softmax_kernel(const float *__restrict__ logits, int B,
-                                                           int E, int k, float *__restrict__ topk_w,
-                                                           int *__restrict__ topk_i) {
-  const int sub = threadIdx.x & 31;
-  const int token = (blockIdx.x * 256 + threadIdx.x) >> 5;
-  const bool live = token < B;
-  const float *row = logits + (size_t)(live ? token : 0) * E;
-  float v[NJ];
-#pragma unroll
-  for (int j = 0; j < NJ; j++) {
-    int e = sub + 32 * j;
-    v[j] = (live && e < E) ? row[e] : -INFINITY;
-  }
+__device__ __forceinline__ void topk_softmax_group(const float (&v)[NJ], int sub, int E, int k,
+                                                   bool live, float *__restrict__ w_out,
+                                                   int *__restrict__ i_out) {
   uint32_t used = 0;
   float pick_v[8];
   int pick_i[8];
@@ -114,7 +52,6 @@ __global__ __launch_bounds__(256) void topk_softmax_kernel(const float *__restri
     }
   }
   if (live && sub == 0) {
-    // softmax over the k picked values: exp in float, sum and divide in double (run.cpp:319-337)
     float ex[8];
     double sum = 0.0;
 #pragma unroll
@@ -125,11 +62,106 @@ __global__ __launch_bounds__(256) void topk_softmax_kernel(const float *__restri
 #pragma unroll
     for (int s = 0; s < 8; s++) {
       if (s < k) {
-        topk_w[(size_t)token * k + s] = (float)((double)ex[s] / sum);
-        topk_i[(size_t)token * k + s] = pick_i[s];
+        w_out[s] = (float)((double)ex[s] / sum);
+        i_out[s] = pick_i[s];
       }
     }
   }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Router GEMM: logits[B,E] = t[B,H] . Wr[E,H]^T + br.  One workgroup = 16 token rows x all experts;
+// its 8 waves split the K loop (k-steps of 32, interleaved), request all their operands up front
+// and reduce through LDS.  With topk_w != nullptr the workgroup also gates its 16 tokens (32
+// lanes per token) while the logits are still in LDS.
+// ------------------------------------------------------------------------------------------------
+constexpr int ROUTER_WAVES = 8;
+constexpr int ROUTER_MAX_STEPS = 6;  // k-steps whose operands a wave keeps in flight at once
+
+template <int NB>  // number of 16-expert column blocks held per wave
+__global__ __launch_bounds__(ROUTER_WAVES * 64) void router_gemm_kernel(
+    const bf16_t *__restrict__ t, const bf16_t *__restrict__ wr, const float *__restrict__ br,
+    float *__restrict__ logits, int B, int H, int E, int k, float *__restrict__ topk_w,
+    int *__restrict__ topk_i) {
+  __shared__ float red[ROUTER_WAVES][16][NB * 16 + 1];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r0 = blockIdx.x * 16;
+  const int arow = min(r0 + (lane & 15), B - 1);
+  const int kq = (lane >> 4) * 8;
+  const bf16_t *ap = t + (size_t)arow * H + kq;
+  f32x4 acc[NB];
+#pragma unroll
+  for (int nb = 0; nb < NB; nb++) acc[nb] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int ksteps = H / 32;
+  for (int ks0 = wave; ks0 < ksteps; ks0 += ROUTER_WAVES * ROUTER_MAX_STEPS) {
+    u32x4 a[ROUTER_MAX_STEPS], b[ROUTER_MAX_STEPS][NB];
+#pragma unroll
+    for (int u = 0; u < ROUTER_MAX_STEPS; u++) {
+      const int ks = min(ks0 + u * ROUTER_WAVES, ksteps - 1);
+      a[u] = *reinterpret_cast<const u32x4 *>(ap + ks * 32);
+#pragma unroll
+      for (int nb = 0; nb < NB; nb++) {
+        int e = min(nb * 16 + (lane & 15), E - 1);
+        b[u][nb] = *reinterpret_cast<const u32x4 *>(wr + (size_t)e * H + ks * 32 + kq);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < ROUTER_MAX_STEPS; u++) {
+      if (ks0 + u * ROUTER_WAVES < ksteps) {
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++)
+          acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a[u]), as_bf16x8(b[u][nb]), acc[nb], 0, 0, 0);
+      }
+    }
+  }
+#pragma unroll
+  for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+    for (int i = 0; i < 4; i++) red[wave][(lane >> 4) * 4 + i][nb * 16 + (lane & 15)] = acc[nb][i];
+  __syncthreads();
+  // 32 lanes per token row: sum the partial products, add the bias, publish, gate
+  const int row = threadIdx.x >> 5, sub = threadIdx.x & 31;
+  const bool live = r0 + row < B;
+  constexpr int NJ = (NB + 1) / 2;
+  float v[NJ];
+#pragma unroll
+  for (int j = 0; j < NJ; j++) {
+    const int e = sub + 32 * j;
+    float x = -INFINITY;
+    if (e < E) {
+      x = 0.f;
+#pragma unroll
+      for (int w = 0; w < ROUTER_WAVES; w++) x += red[w][row][e];
+      if (br) x += br[e];
+      if (live) logits[(size_t)(r0 + row) * E + e] = x;
+    }
+    v[j] = x;
+  }
+  if (topk_w != nullptr) {
+    const size_t o = (size_t)(live ? r0 + row : 0) * k;
+    topk_softmax_group<NJ>(v, sub, E, k, live, topk_w + o, topk_i + o);
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Stand-alone gating from logits in memory: 32 lanes per token, two tokens per wave.
+// ------------------------------------------------------------------------------------------------
+template <int NJ>
+__global__ __launch_bounds__(256) void topk_softmax_kernel(const float *__restrict__ logits, int B,
+                                                           int E, int k, float *__restrict__ topk_w,
+                                                           int *__restrict__ topk_i) {
+  const int sub = threadIdx.x & 31;
+  const int token = (blockIdx.x * 256 + threadIdx.x) >> 5;
+  const bool live = token < B;
+  const float *row = logits + (size_t)(live ? token : 0) * E;
+  float v[NJ];
+#pragma unroll
+  for (int j = 0; j < NJ; j++) {
+    int e = sub + 32 * j;
+    v[j] = (live && e < E) ? row[e] : -INFINITY;
+  }
+  const size_t o = (size_t)(live ? token : 0) * k;
+  topk_softmax_group<NJ>(v, sub, E, k, live, topk_w + o, topk_i + o);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -231,6 +263,23 @@ __global__ __launch_bounds__(SORT_THREADS) void group_sort_kernel(
   }
 }
 
+
+// logits (+ optional gating of the same tokens) in one launch
+int run_router(const void *t, const void *w_router, const float *b_router, float *logits, int B,
+               int H, int E, int k, float *topk_w, int *topk_i, hipStream_t s) {
+  dim3 grid(cdiv(B, 16)), block(ROUTER_WAVES * 64);
+  const bf16_t *tp = (const bf16_t *)t, *wp = (const bf16_t *)w_router;
+  int nb = cdiv(E, 16);
+  TraceScope ts(topk_w ? "router_gemm_topk" : "router_gemm", s);
+  if (nb <= 1) router_gemm_kernel<1><<<grid, block, 0, s>>>(tp, wp, b_router, logits, B, H, E, k, topk_w, topk_i);
+  else if (nb <= 2) router_gemm_kernel<2><<<grid, block, 0, s>>>(tp, wp, b_router, logits, B, H, E, k, topk_w, topk_i);
+  else if (nb <= 4) router_gemm_kernel<4><<<grid, block, 0, s>>>(tp, wp, b_router, logits, B, H, E, k, topk_w, topk_i);
+  else if (nb <= 8) router_gemm_kernel<8><<<grid, block, 0, s>>>(tp, wp, b_router, logits, B, H, E, k, topk_w, topk_i);
+  else router_gemm_kernel<16><<<grid, block, 0, s>>>(tp, wp, b_router, logits, B, H, E, k, topk_w, topk_i);
+  GPTOSS_LAUNCH_CHECK("router_gemm_kernel");
+  return GPTOSS_OK;
+}
+
 }  // namespace gptoss
 
 using namespace gptoss;
@@ -243,18 +292,7 @@ extern "C" int gptoss_router_gemm(const void *t, const void *w_router, const flo
   GPTOSS_REQUIRE(aligned(t, 16) && aligned(w_router, 16), GPTOSS_ERR_ALIGN,
                  "router_gemm: t and w_router must be 16-byte aligned");
   if (B == 0) return GPTOSS_OK;
-  hipStream_t s = (hipStream_t)stream;
-  dim3 grid(cdiv(B, 16)), block(256);
-  const bf16_t *tp = (const bf16_t *)t, *wp = (const bf16_t *)w_router;
-  int nb = cdiv(E, 16);
-  TraceScope ts("router_gemm", s);
-  if (nb <= 1) router_gemm_kernel<1><<<grid, block, 0, s>>>(tp, wp, b_router, logits, B, H, E);
-  else if (nb <= 2) router_gemm_kernel<2><<<grid, block, 0, s>>>(tp, wp, b_router, logits, B, H, E);
-  else if (nb <= 4) router_gemm_kernel<4><<<grid, block, 0, s>>>(tp, wp, b_router, logits, B, H, E);
-  else if (nb <= 8) router_gemm_kernel<8><<<grid, block, 0, s>>>(tp, wp, b_router, logits, B, H, E);
-  else router_gemm_kernel<16><<<grid, block, 0, s>>>(tp, wp, b_router, logits, B, H, E);
-  GPTOSS_LAUNCH_CHECK("router_gemm_kernel");
-  return GPTOSS_OK;
+  return run_router(t, w_router, b_router, logits, B, H, E, 0, nullptr, nullptr, (hipStream_t)stream);
 }
 
 extern "C" int gptoss_moe_max_tiles(int B, int k, int E, int rows_per_tile) {
@@ -263,21 +301,39 @@ extern "C" int gptoss_moe_max_tiles(int B, int k, int E, int rows_per_tile) {
   return (int)(P / rows_per_tile) + E;
 }
 
+static int moe_route_impl(const float *logits, int B, int E, int k, float *topk_w, int *topk_i,
+                          int *expert_offsets, int *sorted_pair_ids, int *inv_perm, int *tiles,
+                          int rows_per_tile, void *stream, bool gate);
+
+// grouping only: topk_i was already written by the fused router kernel
+int gptoss::run_group(int B, int E, int k, float *topk_w, int *topk_i, int *expert_offsets,
+                      int *sorted_pair_ids, int *inv_perm, int *tiles, int rows_per_tile,
+                      hipStream_t s) {
+  return moe_route_impl(nullptr, B, E, k, topk_w, topk_i, expert_offsets, sorted_pair_ids, inv_perm,
+                        tiles, rows_per_tile, s, false);
+}
+
 extern "C" int gptoss_moe_route(const float *logits, int B, int E, int k, float *topk_w,
                                 int *topk_i, int *expert_offsets, int *sorted_pair_ids,
                                 int *inv_perm, int *tiles, int rows_per_tile, void *stream) {
+  return moe_route_impl(logits, B, E, k, topk_w, topk_i, expert_offsets, sorted_pair_ids, inv_perm,
+                        tiles, rows_per_tile, stream, true);
+}
+
+static int moe_route_impl(const float *logits, int B, int E, int k, float *topk_w, int *topk_i,
+                          int *expert_offsets, int *sorted_pair_ids, int *inv_perm, int *tiles,
+                          int rows_per_tile, void *stream, bool gate) {
   GPTOSS_REQUIRE(expert_offsets, GPTOSS_ERR_NULL, "moe_route: null pointer");
-  GPTOSS_REQUIRE(B <= 0 || (logits && topk_w && topk_i && sorted_pair_ids && inv_perm),
+  GPTOSS_REQUIRE(B <= 0 || ((logits || !gate) && topk_w && topk_i && sorted_pair_ids && inv_perm),
                  GPTOSS_ERR_NULL, "moe_route: null pointer");
   GPTOSS_REQUIRE(E >= 1 && E <= 256 && k >= 1 && k <= 8 && k <= E && B >= 0, GPTOSS_ERR_DIM,
                  "moe_route: need 1 <= k <= min(8,E), E <= 256 (B=%d E=%d k=%d)", B, E, k);
   GPTOSS_REQUIRE((long long)B * k < (1ll << 30), GPTOSS_ERR_DIM, "moe_route: B*k too large");
-  bool tile_ok = rows_per_tile == 0 || rows_per_tile == 32 || rows_per_tile == 64 ||
-                 rows_per_tile == 128 || rows_per_tile == 256;
-  GPTOSS_REQUIRE(tile_ok, GPTOSS_ERR_DIM, "moe_route: rows_per_tile must be 0,32,64,128 or 256");
+  bool tile_ok = rows_per_tile >= 0 && rows_per_tile <= 256 && rows_per_tile % 32 == 0;
+  GPTOSS_REQUIRE(tile_ok, GPTOSS_ERR_DIM, "moe_route: rows_per_tile must be 0 or a multiple of 32 up to 256");
   GPTOSS_REQUIRE(rows_per_tile == 0 || tiles, GPTOSS_ERR_NULL, "moe_route: tiles is NULL");
   hipStream_t s = (hipStream_t)stream;
-  if (B > 0) {
+  if (B > 0 && gate) {
     dim3 grid(cdiv(B * 32, 256)), block(256);
     int nj = cdiv(E, 32);
     TraceScope ts("topk_softmax", s);

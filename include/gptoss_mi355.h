@@ -99,7 +99,7 @@ int gptoss_moe_max_tiles(int B, int k, int E, int rows_per_tile);
  * sorted_pair_ids int32 [B*k], inv_perm int32 [B*k] (inv_perm[pair] = its row in the sorted
  * order), tiles int32 [1 + 3*gptoss_moe_max_tiles()] = {n_tiles, (expert,row0,rows)...} cutting
  * every expert's rows into tiles of rows_per_tile (may be NULL with rows_per_tile 0).
- * Needs 1 <= k <= 8, k <= E <= 256, rows_per_tile in {0,32,64,128,256}. */
+ * Needs 1 <= k <= 8, k <= E <= 256, rows_per_tile 0 or a multiple of 32 up to 256. */
 int gptoss_moe_route(const float *logits, int B, int E, int k, float *topk_w, int *topk_i,
                      int *expert_offsets, int *sorted_pair_ids, int *inv_perm, int *tiles,
                      int rows_per_tile, void *stream);

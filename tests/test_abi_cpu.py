@@ -62,7 +62,7 @@ def test_argument_validation_without_gpu(lib):
     assert L.gptoss_router_gemm(p, p, None, p, 4, 250, 8, None) == 2          # H % 32
     assert L.gptoss_moe_route(p, 4, 300, 4, p, p, p, p, p, None, 0, None) == 2  # E > 256
     assert L.gptoss_moe_route(p, 4, 32, 9, p, p, p, p, p, None, 0, None) == 2   # k > 8
-    assert L.gptoss_moe_route(p, 4, 32, 4, p, p, p, p, p, None, 100, None) == 2  # odd tile size
+    assert L.gptoss_moe_route(p, 4, 32, 4, p, p, p, p, p, p, 100, None) == 2     # odd tile size
     assert L.gptoss_pack_weight(p, p, 1, 48, 64, 0, None) == 2                # n_out % 32
     assert L.gptoss_pack_weight(p, p, 1, 32, 64, lib.PACK_GLU, None) == 2     # GLU needs % 64
     assert L.gptoss_kv_cache_write(p, p, p, p, 1, 2, 48, 64, 0, 1, None) == 2  # head_dim
