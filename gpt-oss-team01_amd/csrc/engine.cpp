@@ -187,7 +187,7 @@ int dense_gemm(const bf16_t *A, const bf16_t *W, const float *bias, void *out, i
   g.dense_rows = B;
   g.N = N;
   g.K = K;
-  g.n_col_tiles = cdiv(N, 256);
+  g.n_col_tiles = gemm_col_tiles(N);
   // largest row tile that still gives the 256 CUs at least one workgroup each; the weights of
   // these GEMMs are small enough to be re-read from L2 by the extra row tiles
   static const int sizes[4] = {160, 128, 64, 32};

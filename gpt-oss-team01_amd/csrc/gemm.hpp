@@ -17,7 +17,7 @@ struct GemmParams {
   const int *tiles;    // {n_tiles, (mat,row0,rows)*} or nullptr for a dense problem
   int dense_rows;      // rows of the dense problem when tiles == nullptr
   int N, K;
-  int n_col_tiles;     // cdiv(N, 256)
+  int n_col_tiles;     // gemm_col_tiles(N)
   float limit;         // SwiGLU clamp
 };
 
@@ -27,6 +27,7 @@ int run_gemm(const GemmParams &p, bool gather, int epi, int rows_per_tile, int m
 int run_combine(const float *y2, const float *topk_w, const int *inv_perm, float *out, int B, int H,
                 int k, int accumulate, hipStream_t s);
 int moe_rows_per_tile(int B, int k, int E);
+int gemm_col_tiles(int N);  // column tiles of one workgroup's width
 // moe_route.hip
 int run_router(const void *t, const void *w_router, const float *b_router, float *logits, int B,
                int H, int E, int k, float *topk_w, int *topk_i, hipStream_t s);

@@ -3,4 +3,5 @@
 
 namespace gptoss {
 GPTOSS_GEMM_INSTANTIATE(false)
+int gemm_col_tiles(int N) { return (N + BN - 1) / BN; }
 }  // namespace gptoss

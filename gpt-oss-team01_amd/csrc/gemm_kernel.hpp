@@ -7,18 +7,21 @@
 // expert, i.e. every weight is used by ~128 rows and the kernel is bound by streaming W from
 // HBM.  The design follows from that:
 //   * W is stored in MFMA-fragment order (gptoss_pack_weight): the 1 KB a wave needs for one
-//     32-column x 16-k operand is contiguous, so each wave streams its own columns with
+//     32-column x 16-k operand is contiguous, so each wave streams its own 32 columns with
 //     perfectly coalesced 128-bit loads straight into registers (no LDS hop, no reuse needed:
-//     a workgroup covers all rows of its tile, up to 160, so W is read once);
-//   * the activations (shared by the 4 waves) go through a double-buffered, padded LDS tile; the
+//     a workgroup covers all rows of its tile, up to 160, so W is read from HBM once);
+//   * the activations (shared by the 8 waves) go through a three-stage, padded LDS tile; the
 //     token gather of the reference's pack step is folded into that load;
-//   * a workgroup = 256 virtual columns x up to 160 rows; each wave owns 64 columns as two
-//     B fragments and reuses every A fragment it reads from LDS for two MFMAs;
-//   * work items come from the device-built tile list (expert,row0,rows), mapped so that the
-//     workgroups of one XCD walk consecutive column tiles of the same expert (A stays in that
-//     XCD's L2);
-//   * epilogues: +bias -> fp32, or +bias -> clamped SwiGLU -> bf16 with gate and up of a pair in
-//     the same lane (arranged by the packing order, so no cross-lane traffic).
+//   * a workgroup = 8 waves = 256 columns x up to 160 rows, each wave keeping at most 80
+//     accumulator registers, so two waves share a SIMD: one wave's MFMAs, epilogue or prologue
+//     overlap the other's waits on memory;
+//   * the kernel is persistent (one workgroup per CU); its work items come from the device-built
+//     tile list (expert,row0,rows), mapped so that the workgroups of one XCD walk consecutive
+//     column tiles of the same expert (A stays in that XCD's L2), and the register ring of W keeps
+//     streaming across work items;
+//   * epilogues: +bias -> fp32, or +bias -> clamped SwiGLU -> bf16.  For SwiGLU the packing order
+//     puts the gates of 16 (gate,up) pairs in lanes 0-15 of a wave's columns and their ups in
+//     lanes 16-31, so one cross-lane exchange pairs them.
 #pragma once
 
 #include <type_traits>
@@ -28,10 +31,11 @@
 
 namespace gptoss {
 
-constexpr int GEMM_THREADS = 256;
+constexpr int GEMM_WAVES = 8;
+constexpr int GEMM_THREADS = GEMM_WAVES * 64;
 constexpr int BK = 64;            // k per LDS slab (4 MFMA k-steps)
 constexpr int LDS_ROW = BK + 8;   // padded row length in bf16 elements (144 B)
-constexpr int BN = 256;           // virtual columns per workgroup (4 waves x 64)
+constexpr int BN = GEMM_WAVES * 32;  // columns per workgroup
 
 // MXFP4 operand expansion.  One dword holds the lane's 8 e2m1 codes of a k-step (element j < 4 in
 // the low nibble of byte j, element j >= 4 in the high nibble of byte j-4).  tab[] holds the eight
@@ -78,9 +82,10 @@ __device__ __forceinline__ void static_for(F &&f) {
   }
 }
 
-// Where one wave's two W fragment streams of a work item start.
+// Where one wave's W fragment stream of a work item starts (wave-uniform; each lane adds its own
+// 16 bytes, or 2 scale bytes, when loading).
 struct WStream {
-  const bf16_t *w;           // bf16: first fragment of the wave's first 32-column block
+  const bf16_t *w;           // bf16: first fragment of the wave's 32-column block
   const unsigned char *c;    // MXFP4: codes
   const unsigned char *sc;   // MXFP4: scales
 };
@@ -88,8 +93,8 @@ struct WStream {
 template <bool FP4>
 __device__ __forceinline__ WStream w_stream(const GemmParams &p, int mat, int ct, int wave) {
   const int K = p.K, N = p.N;
-  int n0 = ct * BN + wave * 64;
-  if (n0 >= N) n0 = N - 64;  // idle waves of the last column tile stream a valid block again
+  int n0 = ct * BN + wave * 32;
+  if (n0 >= N) n0 = N - 32;  // idle waves of the last column tile stream a valid block again
   WStream st{nullptr, nullptr, nullptr};
   if (FP4) {
     const int nslab = K / BK;
@@ -100,65 +105,61 @@ __device__ __forceinline__ WStream w_stream(const GemmParams &p, int mat, int ct
   } else {
     st.w = p.W + (size_t)mat * N * K + (size_t)(n0 >> 5) * (K / 16) * 512;
   }
-  return st;  // wave-uniform; each lane adds its own 16 bytes (2 scale bytes) when loading
+  return st;
 }
 
-// Register ring holding NRING slabs of the wave's W operands.
+// Register ring holding NRING slabs of the wave's W operand (bf16: 4 x 16 bytes per lane and
+// slab; MXFP4: 16 bytes of codes + 2 scale bytes).
 template <int NRING, bool FP4>
 struct WRing {
   static constexpr int BQ = FP4 ? 1 : 4;
-  u32x4 b[NRING][2][BQ];
-  uint32_t s[NRING][2];
+  u32x4 b[NRING][BQ];
+  uint32_t s[NRING];
 };
 
 template <int NRING, bool FP4, int R>
-__device__ __forceinline__ void w_load(WRing<NRING, FP4> &ring, const WStream &st, int slab, int K,
-                                       int lane, std::integral_constant<int, R>) {
+__device__ __forceinline__ void w_load(WRing<NRING, FP4> &ring, const WStream &st, int slab, int lane,
+                                       std::integral_constant<int, R>) {
   if (FP4) {
-    const int nslab = K / BK;
-#pragma unroll
-    for (int f = 0; f < 2; f++) {
-      ring.b[R][f][0] = *reinterpret_cast<const u32x4 *>(st.c + (size_t)f * nslab * 1024 +
-                                                         (size_t)slab * 1024 + lane * 16);
-      ring.s[R][f] = *reinterpret_cast<const unsigned short *>(st.sc + (size_t)f * nslab * 64 +
-                                                               (size_t)slab * 64 + (lane & 31) * 2);
-    }
+    ring.b[R][0] = *reinterpret_cast<const u32x4 *>(st.c + (size_t)slab * 1024 + lane * 16);
+    ring.s[R] = *reinterpret_cast<const unsigned short *>(st.sc + (size_t)slab * 64 + (lane & 31) * 2);
   } else {
-    const size_t frag_stride = (size_t)(K / 16) * 512;  // elements between adjacent 32-column blocks
 #pragma unroll
-    for (int f = 0; f < 2; f++)
-#pragma unroll
-      for (int kk = 0; kk < 4; kk++)
-        ring.b[R][f][kk % WRing<NRING, FP4>::BQ] =
-            *reinterpret_cast<const u32x4 *>(st.w + f * frag_stride + (size_t)(slab * 4 + kk) * 512 + lane * 8);
+    for (int kk = 0; kk < 4; kk++)
+      ring.b[R][kk % WRing<NRING, FP4>::BQ] =
+          *reinterpret_cast<const u32x4 *>(st.w + (size_t)(slab * 4 + kk) * 512 + lane * 8);
   }
 }
 
 // One (row tile, column tile) work item with a compile-time number of 32-row blocks, so every
-// loop below is fully unrolled and every global load is unconditional.  On entry the ring holds
-// slabs 0..NRING-2 of this item's W streams; while the last slabs are multiplied the ring is
-// refilled from `next` (the streams of the workgroup's next work item), so the HBM stream of W
+// loop below is fully unrolled and every global load of W is unconditional.  On entry the ring
+// holds slabs 0..NRING-2 of this item's W stream; while the last slabs are multiplied the ring is
+// refilled from `next` (the stream of the workgroup's next work item), so the HBM stream of W
 // never drains between work items.  On exit the ring holds slabs 0..NRING-2 of `next`.
-template <int MB, int NRING, bool GATHER, int EPI, bool FP4>
-__device__ __forceinline__ void gemm_tile(const GemmParams &p, bf16_t *lds, int lds_stage, int mat,
-                                          int row0, int rows, int ct, WRing<NRING, FP4> &ring,
-                                          const WStream &cur, const WStream &next) {
+template <int MB, int MBMAX, int NRING, bool GATHER, int EPI, bool FP4>
+__device__ __forceinline__ void gemm_tile(const GemmParams &p, bf16_t *lds, int mat, int row0, int rows,
+                                          int ct, WRing<NRING, FP4> &ring, const WStream &cur,
+                                          const WStream &next) {
+  constexpr int LDS_STAGE = MBMAX * 32 * LDS_ROW;  // elements per A stage
+  constexpr int D = NRING - 1;                     // slabs of W in flight
+  constexpr int BQ = WRing<NRING, FP4>::BQ;
+  constexpr int APASS = GEMM_THREADS / 8;          // rows moved per pass of the workgroup
+  constexpr int AC = (MB * 32 + APASS - 1) / APASS;  // 16-byte A chunks per thread and slab
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int K = p.K, N = p.N;
-  const int n0_raw = ct * BN + wave * 64;
-  const bool wave_active = n0_raw < N;
-  const int n0 = wave_active ? n0_raw : N - 64;
+  const int n0 = ct * BN + wave * 32;
+  const bool wave_active = n0 < N;
   const int nslab = K / BK;
-  constexpr int D = NRING - 1;  // slabs of W in flight
-  constexpr int BQ = WRing<NRING, FP4>::BQ;
 
-  // ---- A: each thread moves one 16-byte chunk per 32-row block and slab -----------------------
+  // ---- A: the workgroup moves APASS rows x 8 chunks of 16 bytes per pass ----------------------
   const int a_row = tid >> 3, a_kc = tid & 7;
-  uint32_t a_off[MB];
+  uint32_t a_off[AC];
+  bool a_live[AC];
 #pragma unroll
-  for (int i = 0; i < MB; i++) {
-    int r = a_row + 32 * i;
+  for (int i = 0; i < AC; i++) {
+    const int r = a_row + APASS * i;
+    a_live[i] = r < MB * 32;
     int src = GATHER ? 0 : row0;
     if (r < rows) {
       if (GATHER) src = p.row_ids[row0 + r] / p.top_k;
@@ -166,44 +167,36 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, bf16_t *lds, int 
     }
     a_off[i] = (uint32_t)src * (uint32_t)K + a_kc * 8;
   }
-  u32x4 areg[MB];
+  u32x4 areg[AC];
   auto load_a = [&](int s) {
 #pragma unroll
-    for (int i = 0; i < MB; i++) areg[i] = *reinterpret_cast<const u32x4 *>(p.A + a_off[i] + s * BK);
+    for (int i = 0; i < AC; i++)
+      if (a_live[i]) areg[i] = *reinterpret_cast<const u32x4 *>(p.A + a_off[i] + s * BK);
   };
   bf16_t *a_dst = lds + a_row * LDS_ROW + a_kc * 8;
-  auto store_a = [&](int stage) {
+  auto store_a = [&](int stage, bool zero) {
 #pragma unroll
-    for (int i = 0; i < MB; i++)
-      *reinterpret_cast<u32x4 *>(a_dst + stage * lds_stage + 32 * i * LDS_ROW) = areg[i];
+    for (int i = 0; i < AC; i++)
+      if (a_live[i])
+        *reinterpret_cast<u32x4 *>(a_dst + stage * LDS_STAGE + APASS * i * LDS_ROW) =
+            zero ? u32x4{0u, 0u, 0u, 0u} : areg[i];
   };
 
-  auto zero_a = [&](int stage) {
-#pragma unroll
-    for (int i = 0; i < MB; i++)
-      *reinterpret_cast<u32x4 *>(a_dst + stage * lds_stage + 32 * i * LDS_ROW) = u32x4{0u, 0u, 0u, 0u};
-  };
-
-  f32x16 acc[MB][2];
+  f32x16 acc[MB];
 #pragma unroll
   for (int i = 0; i < MB; i++)
 #pragma unroll
-    for (int f = 0; f < 2; f++)
-#pragma unroll
-      for (int r = 0; r < 16; r++) acc[i][f][r] = 0.f;
+    for (int r = 0; r < 16; r++) acc[i][r] = 0.f;
 
   const bf16_t *a_src = lds + (lane & 31) * LDS_ROW + (lane >> 5) * 8;
   bf16x8 af[2][MB];
   auto compute = [&](int stage, auto rsel) {
     constexpr int R = decltype(rsel)::value;
-    const bf16_t *base = a_src + stage * lds_stage;
-    Fp4Table tab[2][2];
+    const bf16_t *base = a_src + stage * LDS_STAGE;
+    Fp4Table tab[2];
     if (FP4) {
-#pragma unroll
-      for (int f = 0; f < 2; f++) {
-        tab[f][0] = fp4_table(ring.s[R][f] & 0xffu);
-        tab[f][1] = fp4_table((ring.s[R][f] >> 8) & 0xffu);
-      }
+      tab[0] = fp4_table(ring.s[R] & 0xffu);
+      tab[1] = fp4_table((ring.s[R] >> 8) & 0xffu);
     }
     // af[0] already holds the fragments of k-step 0 (requested before the previous barrier).  The
     // fragments of k-step kk+1 are requested before the MFMAs of k-step kk are issued, and the
@@ -216,25 +209,18 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, bf16_t *lds, int 
           af[(kk + 1) & 1][i] =
               as_bf16x8(*reinterpret_cast<const u32x4 *>(base + i * 32 * LDS_ROW + (kk + 1) * 16));
       }
-      bf16x8 b0, b1;
-      if (FP4) {
-        b0 = as_bf16x8(fp4_expand(ring.b[R][0][0][kk], tab[0][kk >> 1]));
-        b1 = as_bf16x8(fp4_expand(ring.b[R][1][0][kk], tab[1][kk >> 1]));
-      } else {
-        b0 = as_bf16x8(ring.b[R][0][kk % BQ]);
-        b1 = as_bf16x8(ring.b[R][1][kk % BQ]);
-      }
+      bf16x8 b;
+      if (FP4) b = as_bf16x8(fp4_expand(ring.b[R][0][kk], tab[kk >> 1]));
+      else b = as_bf16x8(ring.b[R][kk % BQ]);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int i = 0; i < MB; i++) {
-        acc[i][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[kk & 1][i], b0, acc[i][0], 0, 0, 0);
-        acc[i][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[kk & 1][i], b1, acc[i][1], 0, 0, 0);
-      }
+      for (int i = 0; i < MB; i++)
+        acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[kk & 1][i], b, acc[i], 0, 0, 0);
       __builtin_amdgcn_sched_barrier(0);
     }
   };
   auto read_first_frags = [&](int stage) {
-    const bf16_t *base = a_src + stage * lds_stage;
+    const bf16_t *base = a_src + stage * LDS_STAGE;
 #pragma unroll
     for (int i = 0; i < MB; i++)
       af[0][i] = as_bf16x8(*reinterpret_cast<const u32x4 *>(base + i * 32 * LDS_ROW));
@@ -248,13 +234,9 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, bf16_t *lds, int 
   const int last = nslab - 1;
   const int padded = (nslab + NRING - 1) / NRING * NRING;
   load_a(0);
-  store_a(0);
-  if (nslab > 1) {
-    load_a(1);
-    store_a(1);
-  } else {
-    zero_a(1);
-  }
+  store_a(0, false);
+  load_a(min(1, last));
+  store_a(1, nslab <= 1);
   load_a(min(2, last));
   __syncthreads();
   read_first_frags(0);
@@ -267,11 +249,10 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, bf16_t *lds, int 
     // then the first slabs of the next item
     const int t = s + D;
     const bool wrap = t >= padded;
-    w_load<NRING, FP4>(ring, wrap ? next : cur, wrap ? t - padded : min(t, last), K, lane, Refill{});
+    w_load<NRING, FP4>(ring, wrap ? next : cur, wrap ? t - padded : min(t, last), lane, Refill{});
     compute(st, rsel);
     const int st1 = (st == 2) ? 0 : st + 1, st2 = (st1 == 2) ? 0 : st1 + 1;
-    if (s + 2 < nslab) store_a(st2);  // rows of slab s+2
-    else zero_a(st2);
+    store_a(st2, s + 2 >= nslab);  // rows of slab s+2 (zeros while padding)
     load_a(min(s + 3, last));
     read_first_frags(st1);
     st = st1;
@@ -283,24 +264,27 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, bf16_t *lds, int 
   if (!wave_active) return;
 
   // ---- epilogue ------------------------------------------------------------------------------
+  // MFMA result layout: lane holds column lane%32, rows (r/4)*8 + (lane/32)*4 + r%4 of each block
   const int c = lane & 31, rsub = (lane >> 5) * 4;
   if (EPI == EPI_SWIGLU) {
+    // columns 0-15 of the wave are the gates of pairs j0..j0+15, columns 16-31 their ups
     const int half_n = N >> 1;
-    const int j = (n0 >> 1) + c;  // pair index: gate = row 2j, up = row 2j+1 of the .bin matrix
-    float bg = 0.f, bu = 0.f;
-    if (p.bias) {
-      bg = p.bias[(size_t)mat * N + 2 * j];
-      bu = p.bias[(size_t)mat * N + 2 * j + 1];
-    }
+    const int j = (n0 >> 1) + (c & 15);  // pair index: gate = row 2j, up = row 2j+1 of the .bin matrix
+    const bool is_up = (c & 16) != 0;
+    const float bias = p.bias ? p.bias[(size_t)mat * N + 2 * j + (is_up ? 1 : 0)] : 0.f;
     bf16_t *o = reinterpret_cast<bf16_t *>(p.out);
     const float L = p.limit;
 #pragma unroll
     for (int i = 0; i < MB; i++) {
 #pragma unroll
       for (int r = 0; r < 16; r++) {
-        int row = i * 32 + (r >> 2) * 8 + rsub + (r & 3);
-        if (row < rows) {
-          float g = acc[i][0][r] + bg, u = acc[i][1][r] + bu;
+        const float mine = acc[i][r] + bias;
+        const float other = __shfl_xor(mine, 16, 64);
+        // gate lanes finish the even result registers, up lanes the odd ones
+        const bool take = ((r & 1) != 0) == is_up;
+        float g = is_up ? other : mine, u = is_up ? mine : other;
+        const int row = i * 32 + (r >> 2) * 8 + rsub + (r & 3);
+        if (take && row < rows) {
           g = fminf(g, L);
           u = fminf(fmaxf(u, -L), L);
           float v = g * (1.0f / (1.0f + expf(-1.702f * g)));
@@ -310,22 +294,19 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, bf16_t *lds, int 
       }
     }
   } else {
+    const int col = n0 + c;
+    const float bv = p.bias ? p.bias[(size_t)mat * N + col] : 0.f;
 #pragma unroll
-    for (int f = 0; f < 2; f++) {
-      const int col = n0 + f * 32 + c;
-      float bv = p.bias ? p.bias[(size_t)mat * N + col] : 0.f;
+    for (int i = 0; i < MB; i++) {
 #pragma unroll
-      for (int i = 0; i < MB; i++) {
-#pragma unroll
-        for (int r = 0; r < 16; r++) {
-          int row = i * 32 + (r >> 2) * 8 + rsub + (r & 3);
-          if (row < rows) {
-            float v = acc[i][f][r] + bv;
-            if (EPI == EPI_F32)
-              reinterpret_cast<float *>(p.out)[(size_t)(row0 + row) * N + col] = v;
-            else
-              reinterpret_cast<bf16_t *>(p.out)[(size_t)(row0 + row) * N + col] = f32_to_bf16(v);
-          }
+      for (int r = 0; r < 16; r++) {
+        const int row = i * 32 + (r >> 2) * 8 + rsub + (r & 3);
+        if (row < rows) {
+          const float v = acc[i][r] + bv;
+          if (EPI == EPI_F32)
+            reinterpret_cast<float *>(p.out)[(size_t)(row0 + row) * N + col] = v;
+          else
+            reinterpret_cast<bf16_t *>(p.out)[(size_t)(row0 + row) * N + col] = f32_to_bf16(v);
         }
       }
     }
@@ -333,22 +314,18 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, bf16_t *lds, int 
 }
 
 // NRING: slabs of W held in registers per wave, NRING-1 of them in flight.
-template <int MBMAX>
-struct RingDepth {
-  static constexpr int value = 3;
-};
+constexpr int GEMM_NRING = 3;
 
-// Persistent kernel: the grid is one workgroup per CU (two for the small-tile kernels); workgroups
-// are dealt round-robin to the 8 XCDs, XCD x owns the x-th contiguous eighth of the work list
-// (consecutive column tiles of the same expert, so that expert's rows stay in that XCD's L2) and
-// its workgroups walk that eighth with a stride of the number of workgroups per XCD.
+// Persistent kernel: the grid is one workgroup of 8 waves per CU; workgroups are dealt round-robin
+// to the 8 XCDs, XCD x owns the x-th contiguous eighth of the work list (consecutive column tiles
+// of the same expert, so that expert's rows stay in that XCD's L2) and its workgroups walk that
+// eighth with a stride of the number of workgroups per XCD.
 template <int MBMAX, bool GATHER, int EPI, bool FP4>
-__global__ __launch_bounds__(GEMM_THREADS) void grouped_gemm_kernel(GemmParams p) {
+__global__ __launch_bounds__(GEMM_THREADS, 2) void grouped_gemm_kernel(GemmParams p) {
   constexpr int BM = MBMAX * 32;
-  constexpr int NRING = RingDepth<MBMAX>::value;
+  constexpr int NRING = GEMM_NRING;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   bf16_t *lds = reinterpret_cast<bf16_t *>(smem_raw);  // [3][BM][LDS_ROW]
-  constexpr int STAGE = BM * LDS_ROW;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
 
@@ -385,7 +362,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void grouped_gemm_kernel(GemmParams p
   WStream cur_w = w_stream<FP4>(p, cur.mat, cur.ct, wave);
   WRing<NRING, FP4> ring;
   static_for<0, NRING - 1>([&](auto r) {
-    w_load<NRING, FP4>(ring, cur_w, min((int)decltype(r)::value, p.K / BK - 1), p.K, lane, r);
+    w_load<NRING, FP4>(ring, cur_w, min((int)decltype(r)::value, p.K / BK - 1), lane, r);
   });
   while (true) {
     const int jn = j + per_xcd;
@@ -399,8 +376,8 @@ __global__ __launch_bounds__(GEMM_THREADS) void grouped_gemm_kernel(GemmParams p
     static_for<1, MBMAX + 1>([&](auto m) {
       constexpr int M = decltype(m)::value;
       if (!done && (mb == M || M == MBMAX)) {
-        gemm_tile<M, NRING, GATHER, EPI, FP4>(p, lds, STAGE, cur.mat, cur.row0, cur.rows, cur.ct, ring,
-                                              cur_w, nxt_w);
+        gemm_tile<M, MBMAX, NRING, GATHER, EPI, FP4>(p, lds, cur.mat, cur.row0, cur.rows, cur.ct, ring,
+                                                     cur_w, nxt_w);
         done = true;
       }
     });
@@ -424,10 +401,8 @@ int launch_gemm(const GemmParams &p, int max_tiles, hipStream_t s) {
     attr_done = true;
   }
   int total = max_tiles * p.n_col_tiles;
-  // one resident workgroup per CU for the large tiles (their registers allow no more), two for
-  // the small ones
-  const int resident = (MBMAX <= 2 ? 2 : 1) * 256;
   int grid = ((total + 7) / 8) * 8;
+  const int resident = 256 * (8 / GEMM_WAVES);  // 8 resident waves (2 per SIMD) per CU
   if (grid > resident) grid = resident;
   if (grid == 0) return GPTOSS_OK;
   {

@@ -52,8 +52,8 @@ __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ 
 
 // Repack row-major [n_out, n_in] matrices into fragment order:
 //   dst[((nb*KS + ks)*64 + lane)*8 + j] = W[row(nb*32 + lane%32)][ks*16 + (lane/32)*8 + j]
-// With GLU pairing, virtual row v of a 64-row wave tile maps to pair (v/64)*32 + v%32, gate for
-// the first 32 virtual rows and up for the second 32.
+// With GLU pairing, virtual row v of a 32-row block maps to pair (v/32)*16 + v%16, gate for the
+// first 16 virtual rows and up for the second 16.
 template <typename SRC>
 __global__ __launch_bounds__(256) void pack_weight_kernel(const SRC *__restrict__ src,
                                                           bf16_t *__restrict__ dst, int n_out,
@@ -68,7 +68,7 @@ __global__ __launch_bounds__(256) void pack_weight_kernel(const SRC *__restrict_
   const int nb = (int)(frag / ksteps), ks = (int)(frag - (size_t)nb * ksteps);
   int v = nb * 32 + (lane & 31);
   int row = v;
-  if (glu) row = 2 * ((v >> 6) * 32 + (v & 31)) + ((v >> 5) & 1);
+  if (glu) row = 2 * ((v >> 5) * 16 + (v & 15)) + ((v >> 4) & 1);
   const SRC *sp = src + ((size_t)mat * n_out + row) * n_in + ks * 16 + (lane >> 5) * 8;
   uint32_t o[4];
 #pragma unroll
@@ -99,7 +99,7 @@ __global__ __launch_bounds__(256) void pack_mxfp4_kernel(const unsigned char *__
   const int nb = (int)(item / nslab), slab = (int)(item - (size_t)nb * nslab);
   int v = nb * 32 + (lane & 31);
   int row = v;
-  if (glu) row = 2 * ((v >> 6) * 32 + (v & 31)) + ((v >> 5) & 1);
+  if (glu) row = 2 * ((v >> 5) * 16 + (v & 15)) + ((v >> 4) & 1);
   const size_t mat_bytes = (size_t)n_out * n_in / 2 + (size_t)n_out * n_in / 32;
   const unsigned char *brow = blocks + ((size_t)mat * n_out + row) * (n_in / 2);
   const unsigned char *srow = scales + ((size_t)mat * n_out + row) * (n_in / 32);
@@ -172,9 +172,8 @@ extern "C" int gptoss_pack_weight(const void *src, void *dst, int n_mat, int n_o
                                   int flags, void *stream) {
   GPTOSS_REQUIRE(src && dst, GPTOSS_ERR_NULL, "pack_weight: null pointer");
   const int glu = (flags & GPTOSS_PACK_GLU) ? 1 : 0;
-  GPTOSS_REQUIRE(n_mat >= 1 && n_out > 0 && n_in > 0 && n_out % (glu ? 64 : 32) == 0 && n_in % 64 == 0,
-                 GPTOSS_ERR_DIM, "pack_weight: need n_out %% %d == 0 and n_in %% 64 == 0 (n_out=%d n_in=%d)",
-                 glu ? 64 : 32, n_out, n_in);
+  GPTOSS_REQUIRE(n_mat >= 1 && n_out > 0 && n_in > 0 && n_out % 32 == 0 && n_in % 64 == 0, GPTOSS_ERR_DIM,
+                 "pack_weight: need n_out %% 32 == 0 and n_in %% 64 == 0 (n_out=%d n_in=%d)", n_out, n_in);
   GPTOSS_REQUIRE(aligned(src, 16) && aligned(dst, 16), GPTOSS_ERR_ALIGN,
                  "pack_weight: pointers must be 16-byte aligned");
   size_t threads = (size_t)(n_out / 32) * (n_in / 16) * 64;
@@ -197,9 +196,8 @@ extern "C" int gptoss_pack_mxfp4(const void *blocks, const void *scales, void *d
                                  int n_out, int n_in, int flags, void *stream) {
   GPTOSS_REQUIRE(blocks && scales && dst, GPTOSS_ERR_NULL, "pack_mxfp4: null pointer");
   const int glu = (flags & GPTOSS_PACK_GLU) ? 1 : 0;
-  GPTOSS_REQUIRE(n_mat >= 1 && n_out > 0 && n_in > 0 && n_out % (glu ? 64 : 32) == 0 && n_in % 64 == 0,
-                 GPTOSS_ERR_DIM, "pack_mxfp4: need n_out %% %d == 0 and n_in %% 64 == 0 (n_out=%d n_in=%d)",
-                 glu ? 64 : 32, n_out, n_in);
+  GPTOSS_REQUIRE(n_mat >= 1 && n_out > 0 && n_in > 0 && n_out % 32 == 0 && n_in % 64 == 0, GPTOSS_ERR_DIM,
+                 "pack_mxfp4: need n_out %% 32 == 0 and n_in %% 64 == 0 (n_out=%d n_in=%d)", n_out, n_in);
   GPTOSS_REQUIRE(aligned(blocks, 4) && aligned(dst, 16), GPTOSS_ERR_ALIGN,
                  "pack_mxfp4: blocks must be 4-byte and dst 16-byte aligned");
   size_t threads = (size_t)(n_out / 32) * (n_in / 64) * 64;

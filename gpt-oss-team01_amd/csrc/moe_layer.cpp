@@ -129,7 +129,7 @@ static int moe_forward_impl(const gptoss_moe_weights *w, const void *t, int B, f
   g1.tiles = ws.tiles;
   g1.N = 2 * I;
   g1.K = H;
-  g1.n_col_tiles = cdiv(2 * I, 256);
+  g1.n_col_tiles = gemm_col_tiles(2 * I);
   g1.limit = w->swiglu_limit;
   rc = run_gemm(g1, true, EPI_SWIGLU, rpt, max_tiles, s);
   if (rc != GPTOSS_OK) return rc;
@@ -143,7 +143,7 @@ static int moe_forward_impl(const gptoss_moe_weights *w, const void *t, int B, f
   g2.tiles = ws.tiles;
   g2.N = H;
   g2.K = I;
-  g2.n_col_tiles = cdiv(H, 256);
+  g2.n_col_tiles = gemm_col_tiles(H);
   rc = run_gemm(g2, false, EPI_F32, rpt, max_tiles, s);
   if (rc != GPTOSS_OK) return rc;
 

@@ -63,7 +63,8 @@ const char *gptoss_trace_name(int i);
 enum {
   GPTOSS_PACK_SRC_FP32 = 1, /* source elements are fp32 (the .bin payload); default bf16 */
   GPTOSS_PACK_GLU = 2       /* rows are interleaved (gate,up) pairs (run.cpp:664-667): reorder them
-                               so a wave holds gate and up of the same pair in one lane */
+                               so a wave holds the gates of 16 pairs in lanes 0-15 and their ups in
+                               lanes 16-31 of its result columns */
 };
 
 /* Bytes of n_mat packed [n_out,n_in] matrices (bf16). */
@@ -71,7 +72,7 @@ size_t gptoss_packed_weight_bytes(int n_mat, int n_out, int n_in);
 
 /* Repack n_mat row-major [n_out,n_in] matrices (device, bf16 or fp32) into MFMA-fragment order.
  * Replaces the host-side transposes of getp-csrc/src/alloc.cpp:27-35,52-59,79-88,112-127,155-170.
- * Needs n_out % 32 == 0 (64 with GPTOSS_PACK_GLU) and n_in % 64 == 0. */
+ * Needs n_out % 32 == 0 and n_in % 64 == 0. */
 int gptoss_pack_weight(const void *src, void *dst, int n_mat, int n_out, int n_in, int flags,
                        void *stream);
 

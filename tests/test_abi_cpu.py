@@ -64,7 +64,7 @@ def test_argument_validation_without_gpu(lib):
     assert L.gptoss_moe_route(p, 4, 32, 9, p, p, p, p, p, None, 0, None) == 2   # k > 8
     assert L.gptoss_moe_route(p, 4, 32, 4, p, p, p, p, p, p, 100, None) == 2     # odd tile size
     assert L.gptoss_pack_weight(p, p, 1, 48, 64, 0, None) == 2                # n_out % 32
-    assert L.gptoss_pack_weight(p, p, 1, 32, 64, lib.PACK_GLU, None) == 2     # GLU needs % 64
+    assert L.gptoss_pack_weight(p, p, 1, 32, 100, lib.PACK_GLU, None) == 2    # n_in % 64
     assert L.gptoss_kv_cache_write(p, p, p, p, 1, 2, 48, 64, 0, 1, None) == 2  # head_dim
     assert L.gptoss_attn_decode(p, p, p, p, None, p, 1, 8, 3, 64, 64, 0, 10, p, 1 << 20, None) == 2
     w = lib.MoeWeights(32, 4, 2880, 2880, 7.0, p.value, p.value, p.value, p.value, p.value, p.value)

@@ -106,11 +106,11 @@ def test_pack_weight_layout(ops):
         row, k0 = nb * 32 + lane % 32, ks * 16 + (lane // 32) * 8
         np.testing.assert_array_equal(wp[m, nb, ks, lane], wn[m, row, k0:k0 + 8])
         np.testing.assert_array_equal(wp32[m, nb, ks, lane], wn[m, row, k0:k0 + 8])
-    # GLU pairing: virtual row v of a 64-row tile -> pair (v//64)*32 + v%32, gate first then up
+    # GLU pairing: virtual row v of a 32-row block -> pair (v//32)*16 + v%16, 16 gates then 16 ups
     wg = ops.pack_weight(w.to(torch.bfloat16).cuda(), glu=True).float().cpu().numpy().reshape(n_mat, N // 32, K // 16, 64, 8)
     for m, nb, ks, lane in [(0, 0, 0, 0), (0, 1, 2, 5), (1, 3, 7, 63), (1, 2, 0, 40)]:
         v = nb * 32 + lane % 32
-        row = 2 * ((v // 64) * 32 + v % 32) + (v // 32) % 2
+        row = 2 * ((v // 32) * 16 + v % 16) + (v // 16) % 2
         k0 = ks * 16 + (lane // 32) * 8
         np.testing.assert_array_equal(wg[m, nb, ks, lane], wn[m, row, k0:k0 + 8])
 
