@@ -59,26 +59,26 @@ __device__ __forceinline__ SeqRange seq_range(int len, int cap, int window, int 
   return r;
 }
 
-// position currently stored in slot s (or -1 if the slot has never been written)
-__device__ __forceinline__ int slot_position(int s, int len, int cap) {
-  int d = len - 1 - s;
-  if (d < 0) return -1;
-  return s + (d / cap) * cap;
-}
-
 template <int D>
 __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
   constexpr int KS = D / 32;   // k-steps of the score MFMA
   constexpr int DB = D / 16;   // 16-row blocks of O^T
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int item = blockIdx.x * 4 + wave;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int item = blockIdx.x * 4 + wave;  // wave-uniform: everything derived from it stays scalar
   const int g = item % p.n_kv;
   const int rest = item / p.n_kv;
   const int b = rest % p.B;
   const int chunk_id = rest / p.B;
   if (chunk_id >= p.max_chunks) return;
-  const SeqRange r = seq_range(p.lens[b], p.cap, p.window, p.chunk, p.max_len);
+  const SeqRange r = seq_range(__builtin_amdgcn_readfirstlane(p.lens[b]), p.cap, p.window, p.chunk, p.max_len);
   if (chunk_id >= r.nchunks) return;
+  // position held by slot s is s + pos_base, or cap less when that would lie beyond the last one
+  const int pos_base = (r.len > 0) ? ((r.len - 1) / p.cap) * p.cap : 0;
+  auto slot_pos = [&](int s) {
+    int pp = s + pos_base;
+    return (pp > r.len - 1) ? pp - p.cap : pp;   // negative for a slot that was never written
+  };
   const int c0 = r.s_begin + chunk_id * p.chunk;
   const int c1 = min(r.s_end, c0 + p.chunk);
   const int n = lane & 15, c = lane >> 4;
@@ -131,8 +131,11 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
   for (int db = 0; db < DB; db++) o[db] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m_run = NEG_BIG, l_run = 0.f;
 
-  auto process = [&](int blk, auto buf) {
+  // EDGE = the block holds slots outside the active positions (first/last block of a range, or
+  // any block of a wrapped ring): only that variant carries the masking code.
+  auto process = [&](int blk, auto buf, auto edge_sel) {
     constexpr int R = decltype(buf)::value;
+    constexpr bool EDGE = decltype(edge_sel)::value;
     // scores for 64 slots x 16 head columns
     f32x4 s4[4];
 #pragma unroll
@@ -146,18 +149,15 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
       }
       s4[tb] = acc;
     }
-    // mask slots outside the active positions (only the edge blocks and wrapped rings need it)
-    const bool edge = (blk < r.t_lo) || (blk + ATT_BLOCK > c1) || (r.len > p.cap);
     float bmax = NEG_BIG;
 #pragma unroll
     for (int tb = 0; tb < 4; tb++)
 #pragma unroll
       for (int i = 0; i < 4; i++) {
         float v = s4[tb][i] * p.scale_log2e;
-        if (edge) {
-          int slot = blk + tb * 16 + c * 4 + i;
-          int pos = slot_position(slot, r.len, p.cap);
-          bool ok = slot < c1 && pos >= r.t_lo;
+        if (EDGE) {
+          const int slot = blk + tb * 16 + c * 4 + i;
+          const bool ok = slot < c1 && slot_pos(slot) >= r.t_lo;
           v = ok ? v : -INFINITY;
         }
         s4[tb][i] = v;
@@ -179,9 +179,11 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
         float p0 = exp2f(s4[grp * 2 + (j >> 1)][(j & 1) * 2] - m_new);
         float p1 = exp2f(s4[grp * 2 + (j >> 1)][(j & 1) * 2 + 1] - m_new);
         psum += p0 + p1;
-        bf16_t h0 = f32_to_bf16(p0), h1 = f32_to_bf16(p1);
-        h[j] = (uint32_t)h0 | ((uint32_t)h1 << 16);
-        l[j] = pack_bf16x2(p0 - bf16_to_f32(h0), p1 - bf16_to_f32(h1));
+        // p is in [0,1]: truncation to bf16 plus the bf16 remainder keeps 16 mantissa bits
+        uint32_t u0 = __float_as_uint(p0), u1 = __float_as_uint(p1);
+        h[j] = (u0 >> 16) | (u1 & 0xffff0000u);
+        float r0 = p0 - __uint_as_float(u0 & 0xffff0000u), r1 = p1 - __uint_as_float(u1 & 0xffff0000u);
+        l[j] = (__float_as_uint(r0) >> 16) | (__float_as_uint(r1) & 0xffff0000u);
       }
       ph[grp] = as_bf16x8(u32x4{h[0], h[1], h[2], h[3]});
       pl[grp] = as_bf16x8(u32x4{l[0], l[1], l[2], l[3]});
@@ -197,14 +199,13 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
 #pragma unroll
       for (int db = 0; db < DB; db++) {
         u32x4 vv = vreg[R][grp][db];
-        if (edge) {
+        if (EDGE) {
           // zero V of inactive slots: never-written cache memory may hold NaN bit patterns
 #pragma unroll
           for (int w = 0; w < 4; w++) {
-            int s_lo = blk + grp * 32 + (w >> 1) * 16 + c * 4 + (w & 1) * 2;
-            int p_lo = slot_position(s_lo, r.len, p.cap), p_hi = slot_position(s_lo + 1, r.len, p.cap);
-            uint32_t keep = ((s_lo < c1 && p_lo >= r.t_lo) ? 0x0000ffffu : 0u) |
-                            ((s_lo + 1 < c1 && p_hi >= r.t_lo) ? 0xffff0000u : 0u);
+            const int s_lo = blk + grp * 32 + (w >> 1) * 16 + c * 4 + (w & 1) * 2;
+            const uint32_t keep = ((s_lo < c1 && slot_pos(s_lo) >= r.t_lo) ? 0x0000ffffu : 0u) |
+                                  ((s_lo + 1 < c1 && slot_pos(s_lo + 1) >= r.t_lo) ? 0xffff0000u : 0u);
             vv[w] &= keep;
           }
         }
@@ -212,6 +213,12 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
         o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, ph[grp], o[db], 0, 0, 0);
         o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pl[grp], o[db], 0, 0, 0);
       }
+  };
+  const bool wrapped = r.len > p.cap;
+  auto step = [&](int blk, auto buf) {
+    const bool edge = wrapped || blk < r.t_lo || blk + ATT_BLOCK > c1;  // wave-uniform
+    if (edge) process(blk, buf, std::true_type{});
+    else process(blk, buf, std::false_type{});
   };
 
   using R0 = std::integral_constant<int, 0>;
@@ -222,11 +229,11 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
     int blk = c0;
     while (true) {
       load_kv(min(blk + ATT_BLOCK, last_blk), R1{});
-      process(blk, R0{});
+      step(blk, R0{});
       blk += ATT_BLOCK;
       if (blk >= c1) break;
       load_kv(min(blk + ATT_BLOCK, last_blk), R0{});
-      process(blk, R1{});
+      step(blk, R1{});
       blk += ATT_BLOCK;
       if (blk >= c1) break;
     }
