@@ -26,6 +26,10 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0         # MI355X HBM3E
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
+# HBM bytes of one GEMM1 launch at the default workload, from two rocprofv3 --pmc runs of this
+# command (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, the factors the 1 GiB copy below calibrates); the
+# summary is kept in profiles/moe_layer_20b_1024tok_and_decode_attention_kernel_stats_and_hbm_traffic.md
+GEMM1_HBM_TRAFFIC_BYTES = (1_102_440 + 23_552) * 1024
 
 
 def parse():
@@ -38,6 +42,7 @@ def parse():
                     help="token slice timed on the CPU baseline (0 = skip)")
     ap.add_argument("--no-attn", action="store_true", help="skip the decode-attention figures")
     ap.add_argument("--no-e2e", action="store_true", help="skip the end-to-end decode figure")
+    ap.add_argument("--no-mxfp4", action="store_true", help="skip the 120B-shape MXFP4 MoE figure")
     return ap.parse_args()
 
 
@@ -115,6 +120,61 @@ def cpu_baseline_moe(torch, state, n_tok):
     return {"value": n_tok / dt, "unit": "tokens/s", "cores": orc.num_threads(), "kind": "port",
             "sample": f"first {n_tok} of the {t.shape[0]} tokens, same tensors, {dt:.1f} s",
             "parity_vs_gpu": {"max_rel": rel_max, "mean_rel": rel_mean}}
+
+
+def bench_moe_mxfp4_120b(ops, torch, steps, warmup):
+    """configs[4]: MoE layer at the GPT-OSS-120B shape with MXFP4 expert weights: 4096 tokens, 128
+    experts, top-4; FP4 codes uniform over the 16 values, one e8m0 scale per 32 inputs with exponent
+    U{-8..0}; router bias Zipf(1.1) over a fixed permutation of the experts."""
+    import numpy as np
+    B, E, H, I, k = 4096, 128, 2880, 2880, 4
+    dev = "cuda"
+    g = torch.Generator(device=dev).manual_seed(99)
+
+    def n(*shape, std=0.02):
+        return (torch.randn(*shape, device=dev, generator=g) * std).to(torch.bfloat16)
+
+    def codes(*shape):
+        return torch.randint(0, 256, shape, device=dev, generator=g, dtype=torch.uint8)
+
+    def scales(*shape):
+        return (127 - torch.randint(0, 9, shape, device=dev, generator=g)).to(torch.uint8)
+
+    ranks = np.random.default_rng(5).permutation(E) + 1
+    br = torch.from_numpy(np.log(1.0 / ranks ** 1.1).astype(np.float32)).to(dev)
+    layers = []
+    for _ in range(2):
+        layers.append(ops.MoeLayerMxfp4(n(E, H), br, codes(E, 2 * I, H // 2), scales(E, 2 * I, H // 32),
+                                        n(E, 2 * I), codes(E, H, I // 2), scales(E, H, I // 32), n(E, H),
+                                        top_k=k, swiglu_limit=7.0, max_tokens=B))
+    t = n(B, H, std=1.0)
+    out = torch.empty(B, H, dtype=torch.float32, device=dev)
+    for i in range(warmup):
+        layers[i % 2].forward(t, out)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        layers[i % 2].forward(t, out)
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    trace = ops.KernelTrace(capacity=8 * steps + 8)
+    with trace:
+        for i in range(steps):
+            layers[i % 2].forward(t, out)
+    kern = trace.summary()
+    counts = np.diff(layers[0].routing_views()[3].cpu().numpy())
+    flops = 2.0 * B * k * H * 3 * I + 2.0 * B * H * E
+    w_bytes = E * 3 * I * H * (0.5 + 1.0 / 32)
+    del layers
+    return {"ms_per_step": round(ms, 4), "tokens_per_s": round(B / ms * 1e3, 1),
+            "tflops": round(flops / ms / 1e9, 1),
+            "mfma_bf16_frac": round(flops / ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4),
+            "weight_mb": round(w_bytes / 1e6, 1), "weight_gbs": round(w_bytes / ms / 1e6, 1),
+            "weight_hbm_frac": round(w_bytes / ms / 1e6 / HBM_PEAK_GBS, 4),
+            "rows_per_expert": {"min": int(counts.min()), "mean": float(counts.mean()), "max": int(counts.max())},
+            "kernels_us": {name: round(v[1] * 1e3, 2) for name, v in kern.items()},
+            "config": "4096 tokens, 128 experts top-4, hidden 2880, intermediate 2880, MXFP4 experts "
+                      "(codes uniform, scale exponent U{-8..0}), Zipf(1.1) router bias, two weight sets alternated"}
 
 
 def bench_attn(ops, torch, steps, warmup):
@@ -226,6 +286,9 @@ def main():
     if not args.no_attn:
         extra["decode_attn"] = bench_attn(ops, torch, max(10, args.steps // 2), args.warmup)
 
+    if not args.no_mxfp4:
+        torch.cuda.empty_cache()
+        extra["moe_120b_mxfp4"] = bench_moe_mxfp4_120b(ops, torch, max(10, args.steps // 2), args.warmup)
     if not args.no_e2e:
         torch.cuda.empty_cache()
         extra["e2e_20b"] = bench_e2e(ops, torch)
@@ -248,9 +311,10 @@ def main():
                    "tokens": args.tokens, "hidden": 2880, "experts": 32, "top_k": 4,
                    "intermediate": 2880, "weights": "bf16 N(0,0.02), two sets alternated",
                    "activations": "bf16 N(0,1)"},
-        "roofline": {"kernel": "grouped_gemm_kernel<8,true,1> (gather + GEMM1 + SwiGLU)",
+        "roofline": {"kernel": "grouped_gemm_kernel<5,true,1,false> (gather + GEMM1 + SwiGLU)",
                      "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": GEMM1_HBM_TRAFFIC_BYTES if args.tokens == 1024 else None,
                      "bytes_per_launch": moe["gemm1_bytes"],
                      "avg_launch_us": round(moe["gemm1_ms"] * 1e3, 2)},
         "cpu_baseline": cpu,

