@@ -19,9 +19,11 @@
 //     tile list (expert,row0,rows), mapped so that the workgroups of one XCD walk consecutive
 //     column tiles of the same expert (A stays in that XCD's L2), and the register ring of W keeps
 //     streaming across work items;
-//   * epilogues: +bias -> fp32, or +bias -> clamped SwiGLU -> bf16.  For SwiGLU the packing order
-//     puts the gates of 16 (gate,up) pairs in lanes 0-15 of a wave's columns and their ups in
-//     lanes 16-31, so one cross-lane exchange pairs them.
+//   * the MFMAs compute the transposed tile (W fragment first), so a lane ends up with one token
+//     row and 16 channels: stores are 8/16 bytes wide, and since the packing order puts the gates
+//     of 16 (gate,up) pairs in channels 0-15 of a wave's block and their ups in channels 16-31,
+//     each pair sits in two registers of the same lane;
+//   * epilogues: +bias -> fp32, or +bias -> clamped SwiGLU -> bf16.
 #pragma once
 
 #include <type_traits>
@@ -215,7 +217,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, bf16_t *lds, int 
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int i = 0; i < MB; i++)
-        acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[kk & 1][i], b, acc[i], 0, 0, 0);
+        acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b, af[kk & 1][i], acc[i], 0, 0, 0);
       __builtin_amdgcn_sched_barrier(0);
     }
   };
@@ -249,7 +251,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, bf16_t *lds, int 
     // then the first slabs of the next item
     const int t = s + D;
     const bool wrap = t >= padded;
-    w_load<NRING, FP4>(ring, wrap ? next : cur, wrap ? t - padded : min(t, last), lane, Refill{});
+    w_load<NRING, FP4>(ring, wrap ? next : cur, min(wrap ? t - padded : t, last), lane, Refill{});
     compute(st, rsel);
     const int st1 = (st == 2) ? 0 : st + 1, st2 = (st1 == 2) ? 0 : st1 + 1;
     store_a(st2, s + 2 >= nslab);  // rows of slab s+2 (zeros while padding)
@@ -264,61 +266,86 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, bf16_t *lds, int 
   if (!wave_active) return;
 
   // ---- epilogue ------------------------------------------------------------------------------
-  // MFMA result layout: lane holds column lane%32, rows (r/4)*8 + (lane/32)*4 + r%4 of each block
-  const int c = lane & 31, rsub = (lane >> 5) * 4;
+  // The MFMAs take the W fragment as their first operand, i.e. they compute the transposed tile:
+  // a lane holds one token row (lane%32 of each 32-row block) and 16 of the wave's 32 output
+  // channels, channel g*8 + h*4 + q in result register g*4 + q (h = lane/32).  Four consecutive
+  // channels of a row are therefore four consecutive registers of one lane, which makes every
+  // store 8 or 16 bytes wide and keeps each (gate, up) pair inside a lane.
+  // Biases are wave-uniform per register and half-wave: they come in through scalar loads, which
+  // do not queue behind the vector loads already in flight for the next item.
+  const int tok = lane & 31;
+  const bool hi = lane >= 32;
+  const int h4 = hi ? 4 : 0;
+  const float *bp = p.bias ? p.bias + (size_t)mat * N + n0 : nullptr;
   if (EPI == EPI_SWIGLU) {
-    // columns 0-15 of the wave are the gates of pairs j0..j0+15, columns 16-31 their ups
+    // channels 0-15 of the wave are the gates of pairs j0..j0+15, channels 16-31 their ups; in the
+    // unpacked matrix pair j is rows 2j (gate) and 2j+1 (up), so its biases are bp[2jj], bp[2jj+1]
     const int half_n = N >> 1;
-    const int j = (n0 >> 1) + (c & 15);  // pair index: gate = row 2j, up = row 2j+1 of the .bin matrix
-    const bool is_up = (c & 16) != 0;
-    const float bias = p.bias ? p.bias[(size_t)mat * N + 2 * j + (is_up ? 1 : 0)] : 0.f;
-    // address = wave-uniform row base (scalar registers) + a 32-bit per-lane element offset
-    bf16_t *o = reinterpret_cast<bf16_t *>(p.out) + (size_t)row0 * half_n;
+    float bg[8], bu[8];
+#pragma unroll
+    for (int g = 0; g < 2; g++)
+#pragma unroll
+      for (int q = 0; q < 4; q++) {
+        const int jlo = g * 8 + q, jhi = jlo + 4;
+        const float g_lo = bp ? bp[2 * jlo] : 0.f, g_hi = bp ? bp[2 * jhi] : 0.f;
+        const float u_lo = bp ? bp[2 * jlo + 1] : 0.f, u_hi = bp ? bp[2 * jhi + 1] : 0.f;
+        bg[g * 4 + q] = hi ? g_hi : g_lo;
+        bu[g * 4 + q] = hi ? u_hi : u_lo;
+      }
+    // address = wave-uniform base (scalar registers) + a 32-bit per-lane element offset
+    bf16_t *o = reinterpret_cast<bf16_t *>(p.out) + (size_t)row0 * half_n + (n0 >> 1);
+    const uint32_t lane_off = (uint32_t)tok * (uint32_t)half_n + (uint32_t)h4;
     const float L = p.limit;
-    // Result registers come in pairs (2q, 2q+1) = two consecutive rows.  The gate lane finishes the
-    // even row and the up lane the odd one: each sends the partner the value it needs and keeps the
-    // other, so every lane evaluates the activation once per pair.
-    const int rlane = rsub + (is_up ? 1 : 0);
-    const uint32_t lane_off = (uint32_t)rlane * (uint32_t)half_n + (uint32_t)j;
+    const int row_lim = rows - tok;  // block i of this lane is a real row iff i*32 < row_lim
 #pragma unroll
     for (int i = 0; i < MB; i++) {
-      float keep[8], recv[8];
+      if (i * 32 < row_lim) {
+        bf16_t *orow = o + (size_t)((uint32_t)(i * 32) * (uint32_t)half_n);
 #pragma unroll
-      for (int q = 0; q < 8; q++) {
-        const float a0 = acc[i][2 * q] + bias, a1 = acc[i][2 * q + 1] + bias;
-        recv[q] = __shfl_xor(is_up ? a0 : a1, 16, 64);
-        keep[q] = is_up ? a1 : a0;
-      }
+        for (int g = 0; g < 2; g++) {
+          float v[4];
 #pragma unroll
-      for (int q = 0; q < 8; q++) {
-        const int rbase = i * 32 + (q >> 1) * 8 + (q & 1) * 2;  // compile-time row of the pair
-        float g = is_up ? recv[q] : keep[q], u = is_up ? keep[q] : recv[q];
-        g = fminf(g, L);
-        u = fminf(fmaxf(u, -L), L);
-        // g * sigmoid(1.702 g) * (u + 1); exp2 and the hardware reciprocal are accurate to a few
-        // ulp of fp32, far inside the bf16 rounding of the result
-        const float e = __builtin_amdgcn_exp2f(-1.702f * 1.4426950408889634f * g);
-        const float v = g * __builtin_amdgcn_rcpf(1.0f + e) * (u + 1.0f);
-        bf16_t *orow = o + (size_t)((uint32_t)rbase * (uint32_t)half_n);
-        if (rlane < rows - rbase) orow[lane_off] = f32_to_bf16(v);
+          for (int q = 0; q < 4; q++) {
+            float gate = acc[i][g * 4 + q] + bg[g * 4 + q];
+            float up = acc[i][(g + 2) * 4 + q] + bu[g * 4 + q];
+            gate = fminf(gate, L);
+            up = fminf(fmaxf(up, -L), L);
+            // gate * sigmoid(1.702 gate) * (up + 1); exp2 and the hardware reciprocal are accurate
+            // to a few ulp of fp32, far inside the bf16 rounding of the result
+            const float e = __builtin_amdgcn_exp2f(-1.702f * 1.4426950408889634f * gate);
+            v[q] = gate * __builtin_amdgcn_rcpf(1.0f + e) * (up + 1.0f);
+          }
+          *reinterpret_cast<u32x2 *>(orow + lane_off + g * 8) =
+              u32x2{pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+        }
       }
-      // one 32-row block at a time: hoisting every exchange first would spill accumulators
-      __builtin_amdgcn_sched_barrier(0);
     }
   } else {
-    const int col = n0 + c;
-    const float bv = p.bias ? p.bias[(size_t)mat * N + col] : 0.f;
+    float bv[16];
+#pragma unroll
+    for (int g = 0; g < 4; g++)
+#pragma unroll
+      for (int q = 0; q < 4; q++) {
+        const float lo = bp ? bp[g * 8 + q] : 0.f, hi_v = bp ? bp[g * 8 + 4 + q] : 0.f;
+        bv[g * 4 + q] = hi ? hi_v : lo;
+      }
+    const uint32_t lane_off = (uint32_t)tok * (uint32_t)N + (uint32_t)h4;
+    const int row_lim = rows - tok;
 #pragma unroll
     for (int i = 0; i < MB; i++) {
+      if (i * 32 < row_lim) {
+        const size_t row_off = (size_t)((uint32_t)(row0 + i * 32) * (uint32_t)N) + n0;
 #pragma unroll
-      for (int r = 0; r < 16; r++) {
-        const int row = i * 32 + (r >> 2) * 8 + rsub + (r & 3);
-        if (row < rows) {
-          const float v = acc[i][r] + bv;
+        for (int g = 0; g < 4; g++) {
+          float v[4];
+#pragma unroll
+          for (int q = 0; q < 4; q++) v[q] = acc[i][g * 4 + q] + bv[g * 4 + q];
           if (EPI == EPI_F32)
-            reinterpret_cast<float *>(p.out)[(size_t)(row0 + row) * N + col] = v;
+            *reinterpret_cast<f32x4 *>(reinterpret_cast<float *>(p.out) + row_off + lane_off + g * 8) =
+                f32x4{v[0], v[1], v[2], v[3]};
           else
-            reinterpret_cast<bf16_t *>(p.out)[(size_t)(row0 + row) * N + col] = f32_to_bf16(v);
+            *reinterpret_cast<u32x2 *>(reinterpret_cast<bf16_t *>(p.out) + row_off + lane_off + g * 8) =
+                u32x2{pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
         }
       }
     }
