@@ -188,16 +188,18 @@ int dense_gemm(const bf16_t *A, const bf16_t *W, const float *bias, void *out, i
   g.N = N;
   g.K = K;
   g.n_col_tiles = gemm_col_tiles(N);
-  // largest row tile that still gives the 256 CUs at least one workgroup each; the weights of
-  // these GEMMs are small enough to be re-read from L2 by the extra row tiles
-  static const int sizes[4] = {160, 128, 64, 32};
-  int rpt = 32;
-  for (int i = 0; i < 4; i++) {
-    rpt = sizes[i];
-    if (rpt == 32) break;
-    if (sizes[i + 1] >= B) continue;  // a smaller tile still holds every row
-    if (cdiv(B, rpt) * g.n_col_tiles >= 256) break;
-  }
+  // Row tile: the smallest size that holds every row of a small batch; for larger batches 96 rows
+  // for the projections (few column tiles: more row tiles keep more CUs busy, fewer re-read the
+  // weights from L2 less often; 96 measured best for N = 2880..5120 at 1024 rows on MI355X) and
+  // 128 rows for the unembedding (hundreds of column tiles, MFMA-bound, 1024 = 8 full tiles).
+  static const int sizes[5] = {32, 64, 96, 128, 160};
+  int rpt = 160;
+  for (int i = 0; i < 5; i++)
+    if (B <= sizes[i]) {
+      rpt = sizes[i];
+      break;
+    }
+  if (B > 96) rpt = (g.n_col_tiles >= 64) ? 128 : 96;
   return run_gemm(g, false, epi, rpt, cdiv(B, rpt), s);
 }
 

@@ -21,7 +21,8 @@ struct GemmParams {
   float limit;         // SwiGLU clamp
 };
 
-// rows_per_tile in {32,64,128,256}; max_tiles bounds the number of (mat,row-tile) items.
+// rows_per_tile in {32,64,96,128,160} (96 only without gather); max_tiles bounds the number of
+// (mat,row-tile) items.
 int run_gemm(const GemmParams &p, bool gather, int epi, int rows_per_tile, int max_tiles,
              hipStream_t s);
 int run_combine(const float *y2, const float *topk_w, const int *inv_perm, float *out, int B, int H,

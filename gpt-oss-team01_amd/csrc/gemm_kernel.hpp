@@ -461,6 +461,7 @@ int launch_gemm(const GemmParams &p, int max_tiles, hipStream_t s) {
   template int launch_gemm<5, true, EPI_SWIGLU, FP4V>(const GemmParams &, int, hipStream_t);   \
   template int launch_gemm<1, false, EPI_F32, FP4V>(const GemmParams &, int, hipStream_t);     \
   template int launch_gemm<2, false, EPI_F32, FP4V>(const GemmParams &, int, hipStream_t);     \
+  template int launch_gemm<3, false, EPI_F32, FP4V>(const GemmParams &, int, hipStream_t);     \
   template int launch_gemm<4, false, EPI_F32, FP4V>(const GemmParams &, int, hipStream_t);     \
   template int launch_gemm<5, false, EPI_F32, FP4V>(const GemmParams &, int, hipStream_t);
 
