@@ -76,7 +76,9 @@ __device__ __forceinline__ void topk_softmax_group(const float (&v)[NJ], int sub
 // lanes per token) while the logits are still in LDS.
 // ------------------------------------------------------------------------------------------------
 constexpr int ROUTER_WAVES = 8;
-constexpr int ROUTER_MAX_STEPS = 6;  // k-steps whose operands a wave keeps in flight at once
+// k-steps whose operands a wave requests before its first MFMA: as many as ~150 registers hold,
+// so that a hidden size of 2880 with up to 32 experts is a single round of loads
+constexpr int router_steps(int nb) { return nb <= 2 ? 12 : (nb <= 4 ? 7 : (nb <= 8 ? 4 : 2)); }
 
 template <int NB>  // number of 16-expert column blocks held per wave
 __global__ __launch_bounds__(ROUTER_WAVES * 64) void router_gemm_kernel(
@@ -92,6 +94,7 @@ __global__ __launch_bounds__(ROUTER_WAVES * 64) void router_gemm_kernel(
   f32x4 acc[NB];
 #pragma unroll
   for (int nb = 0; nb < NB; nb++) acc[nb] = f32x4{0.f, 0.f, 0.f, 0.f};
+  constexpr int ROUTER_MAX_STEPS = router_steps(NB);
   const int ksteps = H / 32;
   for (int ks0 = wave; ks0 < ksteps; ks0 += ROUTER_WAVES * ROUTER_MAX_STEPS) {
     u32x4 a[ROUTER_MAX_STEPS], b[ROUTER_MAX_STEPS][NB];
@@ -183,6 +186,28 @@ __device__ __forceinline__ uint64_t same_expert_mask(int e, bool valid, int nbit
   return mask;
 }
 
+constexpr int SORT_CHUNK = 8;  // 64-pair steps whose expert ids a wave requests at once
+
+// Exclusive prefix sum over up to 256 values held 4 per lane by one wave (lane l owns entries
+// 4l..4l+3); returns the lane's own exclusive prefixes through ex[] and the grand total.
+__device__ __forceinline__ int wave_scan4(const int (&v)[4], int (&ex)[4]) {
+  const int lane = threadIdx.x & 63;
+  int sum = v[0] + v[1] + v[2] + v[3];
+  int inc = sum;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    int o = __shfl_up(inc, d, 64);
+    if (lane >= d) inc += o;
+  }
+  int run = inc - sum;
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    ex[i] = run;
+    run += v[i];
+  }
+  return __shfl(inc, 63, 64);
+}
+
 __global__ __launch_bounds__(SORT_THREADS) void group_sort_kernel(
     const int *__restrict__ topk_i, int P, int E, int nbits, int *__restrict__ expert_offsets,
     int *__restrict__ sorted_pair_ids, int *__restrict__ inv_perm, int *__restrict__ tiles,
@@ -203,18 +228,33 @@ __global__ __launch_bounds__(SORT_THREADS) void group_sort_kernel(
   const int p_end = min(P, p_begin + steps_per_wave * 64);
   int *myhist = hist + wave * E;
 
-  for (int p0 = p_begin; p0 < p_end; p0 += 64) {
-    int p = p0 + lane;
-    int e = (p < p_end) ? topk_i[p] : -1;
-    bool valid = (e >= 0 && e < E);
-    uint64_t mask = same_expert_mask(e, valid, nbits);
-    if (valid && (mask & lt_mask) == 0) myhist[e] += __popcll(mask);
+  // expert ids of SORT_CHUNK steps are requested together, so their latencies overlap
+  auto load_chunk = [&](int p0, int (&e)[SORT_CHUNK]) {
+#pragma unroll
+    for (int u = 0; u < SORT_CHUNK; u++) {
+      const int p = p0 + u * 64 + lane;
+      e[u] = (p < p_end) ? topk_i[p] : -1;
+    }
+  };
+
+  for (int p0 = p_begin; p0 < p_end; p0 += 64 * SORT_CHUNK) {
+    int e[SORT_CHUNK];
+    load_chunk(p0, e);
+#pragma unroll
+    for (int u = 0; u < SORT_CHUNK; u++) {
+      if (p0 + u * 64 < p_end) {  // wave-uniform
+        const bool valid = (e[u] >= 0 && e[u] < E);
+        const uint64_t mask = same_expert_mask(e[u], valid, nbits);
+        if (valid && (mask & lt_mask) == 0) myhist[e[u]] += __popcll(mask);
+      }
+    }
   }
   __syncthreads();
 
   // per expert: exclusive prefix over waves (turns counts into in-expert start ranks), and totals
   for (int e = threadIdx.x; e < E; e += SORT_THREADS) {
     int run = 0;
+#pragma unroll
     for (int w = 0; w < SORT_WAVES; w++) {
       int c = hist[w * E + e];
       hist[w * E + e] = run;
@@ -223,43 +263,61 @@ __global__ __launch_bounds__(SORT_THREADS) void group_sort_kernel(
     total[e] = run;
   }
   __syncthreads();
-  for (int e = threadIdx.x; e <= E; e += SORT_THREADS) {
-    int o = 0;
-    for (int j = 0; j < e; j++) o += total[j];
-    offs[e] = o;
-    expert_offsets[e] = o;
+
+  // expert offsets and first tile of every expert: two prefix sums over E <= 256 entries, wave 0
+  if (wave == 0) {
+    int cnt[4], nt[4], off_ex[4], tile_ex[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const int e = lane * 4 + i;
+      cnt[i] = (e < E) ? total[e] : 0;
+      nt[i] = (rows_per_tile > 0) ? (cnt[i] + rows_per_tile - 1) / rows_per_tile : 0;
+    }
+    const int all = wave_scan4(cnt, off_ex);
+    const int n_tiles = wave_scan4(nt, tile_ex);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const int e = lane * 4 + i;
+      if (e < E) {
+        offs[e] = off_ex[i];
+        expert_offsets[e] = off_ex[i];
+        if (tiles != nullptr && rows_per_tile > 0) {
+          for (int t = 0; t < nt[i]; t++) {
+            int *tp = tiles + 1 + 3 * (tile_ex[i] + t);
+            tp[0] = e;
+            tp[1] = off_ex[i] + t * rows_per_tile;
+            tp[2] = min(rows_per_tile, cnt[i] - t * rows_per_tile);
+          }
+        }
+      }
+    }
+    if (lane == 0) {
+      offs[E] = all;
+      expert_offsets[E] = all;
+      if (tiles != nullptr && rows_per_tile > 0) tiles[0] = n_tiles;
+    }
   }
   __syncthreads();
 
-  if (tiles != nullptr && rows_per_tile > 0) {
-    for (int e = threadIdx.x; e < E; e += SORT_THREADS) {
-      int start = 0;
-      for (int j = 0; j < e; j++) start += (total[j] + rows_per_tile - 1) / rows_per_tile;
-      int rows = total[e];
-      int nt = (rows + rows_per_tile - 1) / rows_per_tile;
-      for (int i = 0; i < nt; i++) {
-        int *tp = tiles + 1 + 3 * (start + i);
-        tp[0] = e;
-        tp[1] = offs[e] + i * rows_per_tile;
-        tp[2] = min(rows_per_tile, rows - i * rows_per_tile);
+  for (int p0 = p_begin; p0 < p_end; p0 += 64 * SORT_CHUNK) {
+    int e[SORT_CHUNK];
+    load_chunk(p0, e);
+#pragma unroll
+    for (int u = 0; u < SORT_CHUNK; u++) {
+      if (p0 + u * 64 < p_end) {
+        const int p = p0 + u * 64 + lane;
+        const bool valid = (e[u] >= 0 && e[u] < E);
+        const uint64_t mask = same_expert_mask(e[u], valid, nbits);
+        if (valid) {
+          const int rank = myhist[e[u]] + __popcll(mask & lt_mask);
+          const int dst = offs[e[u]] + rank;
+          sorted_pair_ids[dst] = p;
+          inv_perm[p] = dst;
+        }
+        // all lanes of the wave have read myhist before the leaders update it (wave-ordered LDS ops)
+        if (valid && (mask & lt_mask) == 0) myhist[e[u]] += __popcll(mask);
       }
-      if (e == E - 1) tiles[0] = start + nt;
     }
-  }
-
-  for (int p0 = p_begin; p0 < p_end; p0 += 64) {
-    int p = p0 + lane;
-    int e = (p < p_end) ? topk_i[p] : -1;
-    bool valid = (e >= 0 && e < E);
-    uint64_t mask = same_expert_mask(e, valid, nbits);
-    if (valid) {
-      int rank = myhist[e] + __popcll(mask & lt_mask);
-      int dst = offs[e] + rank;
-      sorted_pair_ids[dst] = p;
-      inv_perm[p] = dst;
-    }
-    // all lanes of the wave have read myhist before the leaders update it (wave-ordered LDS ops)
-    if (valid && (mask & lt_mask) == 0) myhist[e] += __popcll(mask);
   }
 }
 
