@@ -122,7 +122,21 @@ def cpu_baseline_moe(torch, state, n_tok):
             "parity_vs_gpu": {"max_rel": rel_max, "mean_rel": rel_mean}}
 
 
-def bench_moe_mxfp4_120b(ops, torch, steps, warmup):
+def _dequant_mxfp4(torch, blocks, scales):
+    """e2m1 codes (low nibble = even element) times 2^(scale-127), one scale per 32 inputs -> fp32 on
+    the host, expert by expert (export_model_bin/gpt-oss-20b/export_model_bin.py:66-123)."""
+    lut = torch.tensor([0, .5, 1, 1.5, 2, 3, 4, 6, -0., -.5, -1, -1.5, -2, -3, -4, -6],
+                       device=blocks.device)
+    out = []
+    for e in range(blocks.shape[0]):
+        b = blocks[e]
+        vals = torch.stack([lut[(b & 15).long()], lut[(b >> 4).long()]], -1).reshape(b.shape[0], -1)
+        sc = torch.exp2(scales[e].float() - 127.0).repeat_interleave(32, dim=-1)
+        out.append((vals * sc).cpu())
+    return torch.stack(out).numpy()
+
+
+def bench_moe_mxfp4_120b(ops, torch, steps, warmup, cpu_tokens=0):
     """configs[4]: MoE layer at the GPT-OSS-120B shape with MXFP4 expert weights: 4096 tokens, 128
     experts, top-4; FP4 codes uniform over the 16 values, one e8m0 scale per 32 inputs with exponent
     U{-8..0}; router bias Zipf(1.1) over a fixed permutation of the experts."""
@@ -142,11 +156,14 @@ def bench_moe_mxfp4_120b(ops, torch, steps, warmup):
 
     ranks = np.random.default_rng(5).permutation(E) + 1
     br = torch.from_numpy(np.log(1.0 / ranks ** 1.1).astype(np.float32)).to(dev)
-    layers = []
+    layers, raw = [], None
     for _ in range(2):
-        layers.append(ops.MoeLayerMxfp4(n(E, H), br, codes(E, 2 * I, H // 2), scales(E, 2 * I, H // 32),
-                                        n(E, 2 * I), codes(E, H, I // 2), scales(E, H, I // 32), n(E, H),
-                                        top_k=k, swiglu_limit=7.0, max_tokens=B))
+        w = (n(E, H), br, codes(E, 2 * I, H // 2), scales(E, 2 * I, H // 32), n(E, 2 * I),
+             codes(E, H, I // 2), scales(E, H, I // 32), n(E, H))
+        layers.append(ops.MoeLayerMxfp4(*w, top_k=k, swiglu_limit=7.0, max_tokens=B))
+        if raw is None and cpu_tokens > 0:
+            raw = w
+        del w
     t = n(B, H, std=1.0)
     out = torch.empty(B, H, dtype=torch.float32, device=dev)
     for i in range(warmup):
@@ -165,8 +182,26 @@ def bench_moe_mxfp4_120b(ops, torch, steps, warmup):
     counts = np.diff(layers[0].routing_views()[3].cpu().numpy())
     flops = 2.0 * B * k * H * 3 * I + 2.0 * B * H * E
     w_bytes = E * 3 * I * H * (0.5 + 1.0 / 32)
+    cpu = None
+    if raw is not None:
+        # the oracle's MoE loop on the dequantised fp32 weights, first cpu_tokens tokens
+        from oracle import oracle as orc
+        f = lambda x: x.float().cpu().numpy()
+        w1d, w2d = _dequant_mxfp4(torch, raw[2], raw[3]), _dequant_mxfp4(torch, raw[5], raw[6])
+        tt = f(t[:cpu_tokens])
+        t0 = time.perf_counter()
+        want = orc.moe_layer(tt, f(raw[0]), f(raw[1]), w1d, f(raw[4]), w2d, f(raw[7]), k=k, limit=7.0,
+                             stage=orc.STAGE_SWIGLU)
+        dt = time.perf_counter() - t0
+        got = layers[0].forward(t[:cpu_tokens].contiguous()).cpu().numpy()
+        d = np.abs(got - want)
+        cpu = {"value": round(cpu_tokens / dt, 2), "unit": "tokens/s", "cores": orc.num_threads(), "kind": "port",
+               "sample": f"first {cpu_tokens} tokens on the dequantised fp32 weights, {dt:.1f} s",
+               "parity_vs_gpu": {"max_rel": float(d.max() / np.abs(want).max()),
+                                 "mean_rel": float(d.mean() / np.abs(want).mean())}}
+        del w1d, w2d, raw
     del layers
-    return {"ms_per_step": round(ms, 4), "tokens_per_s": round(B / ms * 1e3, 1),
+    return {"cpu_baseline": cpu, "ms_per_step": round(ms, 4), "tokens_per_s": round(B / ms * 1e3, 1),
             "tflops": round(flops / ms / 1e9, 1),
             "mfma_bf16_frac": round(flops / ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4),
             "weight_mb": round(w_bytes / 1e6, 1), "weight_gbs": round(w_bytes / ms / 1e6, 1),
@@ -208,6 +243,43 @@ def bench_attn(ops, torch, steps, warmup):
         res[name] = {"us": round(ms * 1e3, 1), "kv_mb": round(kv_bytes / 1e6, 1),
                      "gbs": round(kv_bytes / ms / 1e6, 1),
                      "hbm_frac": round(kv_bytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
+    return res
+
+
+def cpu_baseline_attn(ops, torch, n_seq=32):
+    """configs[2] on the host: the oracle's restatement of run.cpp:562-607 (OpenMP over sequence and
+    head) on n_seq sequences of the same shape, with the GPU result of the same tensors beside it."""
+    import numpy as np
+    from oracle import oracle as orc
+    n_q, n_kv, D, S = 64, 8, 64, 4096
+    rng = np.random.default_rng(1)
+    lens_np = rng.integers(512, S + 1, size=n_seq).astype(np.int32)
+    g = torch.Generator(device="cuda").manual_seed(7)
+    k_rows = torch.randn(n_seq, S, n_kv, D, device="cuda", generator=g).to(torch.bfloat16)
+    v_rows = torch.randn(n_seq, S, n_kv, D, device="cuda", generator=g).to(torch.bfloat16)
+    q = torch.randn(n_seq, n_q, D, device="cuda", generator=g)
+    sinks = torch.randn(n_q, device="cuda", generator=g)
+    cache = ops.KVCache(n_seq, n_kv, D, S)
+    cache.write(k_rows, v_rows, 0)
+    attn = ops.AttnDecode(n_seq, n_q, n_kv, D, S)
+    lens = torch.from_numpy(lens_np).cuda()
+    kf, vf = k_rows.float().cpu().numpy(), v_rows.float().cpu().numpy()
+    qf, sf = q.cpu().numpy(), sinks.cpu().numpy()
+    res = {}
+    for name, window in (("full", 0), ("window128", 128)):
+        got = attn.forward(q, cache, lens, sinks, window=window).float().cpu().numpy()
+        t0 = time.perf_counter()
+        want = orc.attn_decode(qf, kf, vf, lens_np, sf, window=window)
+        dt = time.perf_counter() - t0
+        act = np.minimum(lens_np, window) if window else lens_np
+        kv_bytes = int(act.sum()) * n_kv * D * 2 * 2
+        d = np.abs(got - want)
+        res[name] = {"gbs": round(kv_bytes / dt / 1e9, 2), "seconds": round(dt, 3),
+                     "parity_vs_gpu": {"max_rel": float(d.max() / np.abs(want).max()),
+                                       "mean_rel": float(d.mean() / np.abs(want).mean())}}
+    res["cores"] = orc.num_threads()
+    res["kind"] = "port"
+    res["sample"] = f"{n_seq} sequences of the same shape (lengths U[512,4096]), bf16 KV bytes per second"
     return res
 
 
@@ -285,14 +357,25 @@ def main():
              "gemm1_tflops": round(moe["gemm1_flops"] / moe["gemm1_ms"] / 1e9, 1)}
     if not args.no_attn:
         extra["decode_attn"] = bench_attn(ops, torch, max(10, args.steps // 2), args.warmup)
+        if args.cpu_tokens > 0:
+            extra["decode_attn"]["cpu_baseline"] = cpu_baseline_attn(ops, torch)
 
     if not args.no_mxfp4:
         torch.cuda.empty_cache()
-        extra["moe_120b_mxfp4"] = bench_moe_mxfp4_120b(ops, torch, max(10, args.steps // 2), args.warmup)
+        extra["moe_120b_mxfp4"] = bench_moe_mxfp4_120b(ops, torch, max(10, args.steps // 2), args.warmup,
+                                                       cpu_tokens=min(64, args.cpu_tokens))
     if not args.no_e2e:
         torch.cuda.empty_cache()
         extra["e2e_20b"] = bench_e2e(ops, torch)
 
+    if cpu is not None and "e2e_20b" in extra:
+        # whole-model CPU figure: not run (84 GB of fp32 weights, minutes per token); scaled from the
+        # measured CPU MoE-layer rate by FLOPs per token (24 blocks of MoE 199 + projections 53 MFLOP,
+        # plus the 1158 MFLOP unembedding)
+        per_tok_s = (1.0 / cpu["value"]) * (24 * (199.1 + 53.1) + 1158.3) / 199.1
+        extra["e2e_20b"]["cpu_baseline"] = {"value": round(1.0 / per_tok_s, 2), "unit": "tokens/s",
+                                            "cores": cpu["cores"], "kind": "port",
+                                            "sample": "extrapolated from the measured CPU MoE-layer rate by FLOPs per token"}
     achieved = moe["gemm1_bytes"] / moe["gemm1_ms"] / 1e6
     line = {
         "metric": "MoE-layer tokens/s (GPT-OSS-20B layer shape, 1024 tokens, 1 GPU)",
