@@ -269,27 +269,59 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
   }
 }
 
-// Merge the chunk partials of one (sequence, q head) with the sink logit.
+// Merge the chunk partials of one (sequence, q head) with the sink logit.  One thread owns four
+// consecutive output elements; the chunk loop is unrolled in groups of ATT_RED_UNROLL whose loads
+// are all requested before the first use.
+constexpr int ATT_RED_UNROLL = 4;
+
 template <int D>
 __global__ __launch_bounds__(256) void attn_reduce_kernel(AttnParams p) {
-  const int pair = blockIdx.x * (256 / D) + threadIdx.x / D;  // (b, head)
-  const int d = threadIdx.x % D;
+  constexpr int TPP = D / 4;  // threads per (b, head)
+  const int pair = blockIdx.x * (256 / TPP) + threadIdx.x / TPP;
+  const int d4 = (threadIdx.x % TPP) * 4;
   if (pair >= p.B * p.n_q) return;
   const int b = pair / p.n_q, hq = pair - b * p.n_q;
   const SeqRange r = seq_range(p.lens[b], p.cap, p.window, p.chunk, p.max_len);
   if (r.nchunks <= 1) return;  // already finished by the first kernel
   const float sink2 = p.sinks ? p.sinks[hq] * 1.4426950408889634f : -INFINITY;
+  const size_t slot0 = (size_t)b * p.max_chunks * p.n_q + hq;
+  const size_t slot_stride = p.n_q;
   float M = sink2;
-  for (int ch = 0; ch < r.nchunks; ch++)
-    M = fmaxf(M, p.part_ml[(((size_t)b * p.max_chunks + ch) * p.n_q + hq) * 2]);
-  float denom = exp2f(sink2 - M), acc = 0.f;
-  for (int ch = 0; ch < r.nchunks; ch++) {
-    size_t slot = ((size_t)b * p.max_chunks + ch) * p.n_q + hq;
-    float w = exp2f(p.part_ml[slot * 2] - M);
-    denom += p.part_ml[slot * 2 + 1] * w;
-    acc += p.part_o[slot * D + d] * w;
+  for (int c0 = 0; c0 < r.nchunks; c0 += ATT_RED_UNROLL) {
+    float m[ATT_RED_UNROLL];
+#pragma unroll
+    for (int u = 0; u < ATT_RED_UNROLL; u++)
+      m[u] = (c0 + u < r.nchunks) ? p.part_ml[(slot0 + (size_t)(c0 + u) * slot_stride) * 2] : -INFINITY;
+#pragma unroll
+    for (int u = 0; u < ATT_RED_UNROLL; u++) M = fmaxf(M, m[u]);
   }
-  p.out[((size_t)b * p.n_q + hq) * D + d] = f32_to_bf16(denom > 0.f ? acc / denom : 0.f);
+  float denom = exp2f(sink2 - M);
+  f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int c0 = 0; c0 < r.nchunks; c0 += ATT_RED_UNROLL) {
+    float m[ATT_RED_UNROLL], l[ATT_RED_UNROLL];
+    f32x4 o[ATT_RED_UNROLL];
+#pragma unroll
+    for (int u = 0; u < ATT_RED_UNROLL; u++) {
+      const bool ok = c0 + u < r.nchunks;
+      const size_t slot = slot0 + (size_t)(ok ? c0 + u : 0) * slot_stride;
+      m[u] = ok ? p.part_ml[slot * 2] : -INFINITY;
+      l[u] = ok ? p.part_ml[slot * 2 + 1] : 0.f;
+      o[u] = *reinterpret_cast<const f32x4 *>(p.part_o + slot * D + d4);
+    }
+    // chunks are merged in ascending order, so the result does not depend on the unroll width
+#pragma unroll
+    for (int u = 0; u < ATT_RED_UNROLL; u++) {
+      if (c0 + u < r.nchunks) {
+        const float w = exp2f(m[u] - M);
+        denom += l[u] * w;
+#pragma unroll
+        for (int q = 0; q < 4; q++) acc[q] += o[u][q] * w;
+      }
+    }
+  }
+  u32x2 pk = u32x2{pack_bf16x2(denom > 0.f ? acc[0] / denom : 0.f, denom > 0.f ? acc[1] / denom : 0.f),
+                   pack_bf16x2(denom > 0.f ? acc[2] / denom : 0.f, denom > 0.f ? acc[3] / denom : 0.f)};
+  *reinterpret_cast<u32x2 *>(p.out + ((size_t)b * p.n_q + hq) * D + d4) = pk;
 }
 
 // Bulk cache write: rows [B, n_tok, n_kv, D] -> K [B, n_kv, cap, D], V in 32-slot operand blocks.
@@ -423,7 +455,7 @@ extern "C" int gptoss_attn_decode(const float *q, const void *k_cache, const voi
   }
   GPTOSS_LAUNCH_CHECK("attn_decode_kernel");
   if (pl.max_chunks > 1) {
-    int per_block = 256 / head_dim;
+    int per_block = 256 / (head_dim / 4);
     int rgrid = (B * n_q + per_block - 1) / per_block;
     TraceScope ts("attn_reduce", s);
     if (head_dim == 64) attn_reduce_kernel<64><<<rgrid, 256, 0, s>>>(p);
