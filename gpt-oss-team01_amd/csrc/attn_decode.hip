@@ -85,25 +85,6 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
   const int G = p.G;
   const int head = g * G + min(n, G - 1);
 
-  // ---- Q^T operand, split into bf16 hi and lo parts -----------------------------------------
-  bf16x8 qh[KS], ql[KS];
-  {
-    const float *qp = p.q + ((size_t)b * p.n_q + head) * D + c * KS * 8;
-#pragma unroll
-    for (int s = 0; s < KS; s++) {
-      uint32_t h[4], l[4];
-#pragma unroll
-      for (int j = 0; j < 4; j++) {
-        float x0 = (n < G) ? qp[s * 8 + 2 * j] : 0.f, x1 = (n < G) ? qp[s * 8 + 2 * j + 1] : 0.f;
-        bf16_t h0 = f32_to_bf16(x0), h1 = f32_to_bf16(x1);
-        h[j] = (uint32_t)h0 | ((uint32_t)h1 << 16);
-        l[j] = pack_bf16x2(x0 - bf16_to_f32(h0), x1 - bf16_to_f32(h1));
-      }
-      qh[s] = as_bf16x8(u32x4{h[0], h[1], h[2], h[3]});
-      ql[s] = as_bf16x8(u32x4{l[0], l[1], l[2], l[3]});
-    }
-  }
-
   const bf16_t *kbase = p.kc + ((size_t)(b * p.n_kv + g) * p.cap) * D;
   const bf16_t *vbase = p.vc + ((size_t)(b * p.n_kv + g) * p.cap) * D;
   // lane's K bytes for slot block `blk`: slot blk + tb*16 + n, d chunk c*KS*8 .. +KS*8
@@ -125,6 +106,31 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
         vreg[R][grp][db] = *reinterpret_cast<const u32x4 *>(
             vbase + ((size_t)((blk >> 5) + grp) * DB + db) * 512 + v_lane);
   };
+
+  // the first K/V block is requested before anything waits on q, so the cache stream of a work
+  // item starts one memory latency earlier
+  using R0 = std::integral_constant<int, 0>;
+  using R1 = std::integral_constant<int, 1>;
+  if (c1 > c0) load_kv(c0, R0{});
+
+  // ---- Q^T operand, split into bf16 hi and lo parts -----------------------------------------
+  bf16x8 qh[KS], ql[KS];
+  {
+    const float *qp = p.q + ((size_t)b * p.n_q + head) * D + c * KS * 8;
+#pragma unroll
+    for (int s = 0; s < KS; s++) {
+      uint32_t h[4], l[4];
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        float x0 = (n < G) ? qp[s * 8 + 2 * j] : 0.f, x1 = (n < G) ? qp[s * 8 + 2 * j + 1] : 0.f;
+        bf16_t h0 = f32_to_bf16(x0), h1 = f32_to_bf16(x1);
+        h[j] = (uint32_t)h0 | ((uint32_t)h1 << 16);
+        l[j] = pack_bf16x2(x0 - bf16_to_f32(h0), x1 - bf16_to_f32(h1));
+      }
+      qh[s] = as_bf16x8(u32x4{h[0], h[1], h[2], h[3]});
+      ql[s] = as_bf16x8(u32x4{l[0], l[1], l[2], l[3]});
+    }
+  }
 
   f32x4 o[DB];
 #pragma unroll
@@ -221,11 +227,8 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
     else process(blk, buf, std::false_type{});
   };
 
-  using R0 = std::integral_constant<int, 0>;
-  using R1 = std::integral_constant<int, 1>;
   const int last_blk = max(c0, ((c1 - 1) & ~(ATT_BLOCK - 1)));
   if (c1 > c0) {
-    load_kv(c0, R0{});
     int blk = c0;
     while (true) {
       load_kv(min(blk + ATT_BLOCK, last_blk), R1{});

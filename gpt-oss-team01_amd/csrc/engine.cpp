@@ -10,6 +10,7 @@
 #include "common.hpp"
 #include "gemm.hpp"
 #include "glue.hpp"
+#include "precise.hpp"
 
 #ifndef M_PI
 #define M_PI 3.14159265358979323846
@@ -58,6 +59,15 @@ struct gptoss_engine {
   void *moe_ws, *attn_ws;
   size_t moe_ws_bytes, attn_ws_bytes;
   size_t device_bytes;
+  // fp32-faithful mode (GPTOSS_ENGINE_PRECISE): the .bin payload as it is, fp32 KV caches and
+  // fp32 intermediates
+  struct Precise {
+    float *payload;  // whole fp32 payload, tensor offsets below in floats
+    size_t emb, unemb, attn_norm, mlp_norm, fin, w_qkv, b_qkv, w_o, b_o, sinks, w_router, b_router, w1, b1, w2, b2;
+    float *kc, *vc;  // [L, B, max_seq, kv_dim]
+    float *t, *attn, *att, *router, *topk_w, *mlp1, *act, *mlp2;
+    int *topk_i;
+  } pr;
 };
 
 namespace {
@@ -214,14 +224,127 @@ void destroy(gptoss_engine *e) {
 
 }  // namespace
 
+// ---- fp32-faithful mode ------------------------------------------------------------------------
+static int create_precise(gptoss_engine *e, Builder &b, const float *host_weights) {
+  const gptoss_config &c = e->cfg;
+  const size_t H = c.hidden_dim, V = c.vocab_size, L = c.n_layers, E = c.n_experts, k = c.experts_per_token;
+  const size_t D = c.head_dim, nq = c.n_attn_heads, nkv = c.n_kv_heads, I = c.intermediate_dim;
+  const size_t qkv_dim = (nq + 2 * nkv) * D, B = e->max_batch, S = e->max_seq;
+  gptoss_engine::Precise &pr = e->pr;
+  // tensor order of the .bin payload (reference run.cpp:194-233)
+  size_t off = 0;
+  auto take = [&](size_t n) {
+    size_t o = off;
+    off += n;
+    return o;
+  };
+  pr.emb = take(V * H);
+  pr.unemb = take(V * H);
+  pr.attn_norm = take(L * H);
+  pr.mlp_norm = take(L * H);
+  pr.fin = take(H);
+  pr.w_qkv = take(L * qkv_dim * H);
+  pr.b_qkv = take(L * qkv_dim);
+  pr.w_o = take(L * H * nq * D);
+  pr.b_o = take(L * H);
+  pr.sinks = take(L * nq);
+  pr.w_router = take(L * E * H);
+  pr.b_router = take(L * E);
+  pr.w1 = take(L * E * 2 * I * H);
+  pr.b1 = take(L * E * 2 * I);
+  pr.w2 = take(L * E * H * I);
+  pr.b2 = take(L * E * H);
+  pr.payload = b.alloc<float>(off);
+  if (b.ok()) b.hip(hipMemcpy(pr.payload, host_weights, off * sizeof(float), hipMemcpyHostToDevice), "H2D");
+  const size_t kv_dim = nkv * D;
+  pr.kc = b.alloc<float>(L * B * S * kv_dim);
+  pr.vc = b.alloc<float>(L * B * S * kv_dim);
+  std::vector<float> cs, sn;
+  rope_tables(c, (int)S, cs, sn);
+  e->cos_t = b.alloc<float>(cs.size());
+  e->sin_t = b.alloc<float>(sn.size());
+  if (b.ok()) {
+    b.hip(hipMemcpy(e->cos_t, cs.data(), cs.size() * 4, hipMemcpyHostToDevice), "H2D");
+    b.hip(hipMemcpy(e->sin_t, sn.data(), sn.size() * 4, hipMemcpyHostToDevice), "H2D");
+  }
+  e->d_tokens = b.alloc<int>(B);
+  e->d_next = b.alloc<int>(B);
+  e->d_lens = nullptr;
+  e->x = b.alloc<float>(B * H);
+  e->t = b.alloc<bf16_t>(B * H);  // written by the norm kernel, unused
+  pr.t = b.alloc<float>(B * H);
+  e->qkv = b.alloc<float>(B * qkv_dim);
+  e->q = b.alloc<float>(B * nq * D);
+  pr.attn = b.alloc<float>(B * nq * D);
+  pr.att = b.alloc<float>(B * nq * (S + 2));
+  e->tb2 = b.alloc<float>(B * H);
+  pr.router = b.alloc<float>(B * E);
+  pr.topk_w = b.alloc<float>(B * k);
+  pr.topk_i = b.alloc<int>(B * k);
+  pr.mlp1 = b.alloc<float>(B * k * 2 * I);
+  pr.act = b.alloc<float>(B * k * I);
+  pr.mlp2 = b.alloc<float>(B * k * H);
+  e->logits = b.alloc<float>(B * V);
+  if (b.ok()) b.hip(hipStreamSynchronize(e->stream), "sync");
+  return b.rc;
+}
+
+// one lock-step position with the arithmetic of the reference CPU forward (run.cpp:501-717)
+static int precise_step(gptoss_engine *e, int pos, int B) {
+  const gptoss_config &c = e->cfg;
+  const int H = c.hidden_dim, V = c.vocab_size, L = c.n_layers, E = c.n_experts, k = c.experts_per_token;
+  const int D = c.head_dim, nq = c.n_attn_heads, nkv = c.n_kv_heads, I = c.intermediate_dim;
+  const int qkv_dim = (nq + 2 * nkv) * D, S = e->max_seq;
+  const size_t kv_dim = (size_t)nkv * D;
+  hipStream_t s = e->stream;
+  const gptoss_engine::Precise &pr = e->pr;
+  const float *W = pr.payload;
+  int rc;
+#define STEP(call)                   \
+  do {                               \
+    rc = (call);                     \
+    if (rc != GPTOSS_OK) return rc;  \
+  } while (0)
+  STEP(precise_embedding(W + pr.emb, e->d_tokens, e->x, B, H, V, s));
+  for (int l = 0; l < L; l++) {
+    STEP(run_rmsnorm(e->x, nullptr, W + pr.attn_norm + (size_t)l * H, e->t, pr.t, B, H, s));
+    STEP(precise_matmul(e->qkv, pr.t, W + pr.w_qkv + (size_t)l * qkv_dim * H, W + pr.b_qkv + (size_t)l * qkv_dim,
+                        nullptr, B, H, qkv_dim, 1, s));
+    float *kc = pr.kc + (size_t)l * e->max_batch * S * kv_dim, *vc = pr.vc + (size_t)l * e->max_batch * S * kv_dim;
+    STEP(precise_rope_store(e->qkv, e->q, kc, vc, e->cos_t, e->sin_t, B, nq, nkv, D, S, pos, s));
+    const int window = (c.sliding_window > 0 && l % 2 == 0) ? c.sliding_window : 0;
+    STEP(precise_attn(e->q, kc, vc, W + pr.sinks + (size_t)l * nq, pr.att, pr.attn, B, nq, nkv, D, S, pos,
+                      window, s));
+    STEP(precise_matmul(e->tb2, pr.attn, W + pr.w_o + (size_t)l * H * nq * D, W + pr.b_o + (size_t)l * H, nullptr,
+                        B, nq * D, H, 1, s));
+    STEP(precise_add(e->x, e->tb2, (size_t)B * H, s));
+    STEP(run_rmsnorm(e->x, nullptr, W + pr.mlp_norm + (size_t)l * H, e->t, pr.t, B, H, s));
+    STEP(precise_matmul(pr.router, pr.t, W + pr.w_router + (size_t)l * E * H, W + pr.b_router + (size_t)l * E,
+                        nullptr, B, H, E, 1, s));
+    STEP(run_topk_softmax(pr.router, B, E, k, pr.topk_w, pr.topk_i, s));
+    // one row per (token, slot): the slot's expert selects the matrix
+    STEP(precise_matmul(pr.mlp1, pr.t, W + pr.w1 + (size_t)l * E * 2 * I * H, W + pr.b1 + (size_t)l * E * 2 * I,
+                        pr.topk_i, B * k, H, 2 * I, k, s));
+    STEP(precise_swiglu(pr.mlp1, pr.act, B * k, I, c.swiglu_limit, s));
+    STEP(precise_matmul(pr.mlp2, pr.act, W + pr.w2 + (size_t)l * E * H * I, W + pr.b2 + (size_t)l * E * H,
+                        pr.topk_i, B * k, I, H, 1, s));
+    STEP(precise_moe_agg(pr.mlp2, pr.topk_w, pr.topk_i, e->x, B, H, k, s));
+  }
+  STEP(run_rmsnorm(e->x, nullptr, W + pr.fin, e->t, pr.t, B, H, s));
+  STEP(precise_matmul(e->logits, pr.t, W + pr.unemb, nullptr, nullptr, B, H, V, 1, s));
+#undef STEP
+  return GPTOSS_OK;
+}
+
 extern "C" int gptoss_engine_create(const gptoss_config *cfg, const float *host_weights, int max_batch,
                                     int max_seq, int flags, uint64_t seed, gptoss_engine **out) {
   GPTOSS_REQUIRE(cfg && out, GPTOSS_ERR_NULL, "engine_create: null pointer");
   *out = nullptr;
   const bool synthetic = (flags & GPTOSS_ENGINE_SYNTHETIC) != 0;
   GPTOSS_REQUIRE(synthetic || host_weights, GPTOSS_ERR_NULL, "engine_create: host_weights is NULL");
-  GPTOSS_REQUIRE(!(flags & GPTOSS_ENGINE_PRECISE), GPTOSS_ERR_STATE,
-                 "engine_create: GPTOSS_ENGINE_PRECISE is not available in this build");
+  const bool precise = (flags & GPTOSS_ENGINE_PRECISE) != 0;
+  GPTOSS_REQUIRE(!(precise && synthetic), GPTOSS_ERR_STATE,
+                 "engine_create: GPTOSS_ENGINE_PRECISE needs host weights (not GPTOSS_ENGINE_SYNTHETIC)");
   const gptoss_config &c = *cfg;
   const int H = c.hidden_dim, V = c.vocab_size, L = c.n_layers, E = c.n_experts, k = c.experts_per_token;
   const int D = c.head_dim, nq = c.n_attn_heads, nkv = c.n_kv_heads, I = c.intermediate_dim;
@@ -252,6 +375,15 @@ extern "C" int gptoss_engine_create(const gptoss_config *cfg, const float *host_
   b.hip(hipStreamCreate(&e->stream), "hipStreamCreate");
   b.hip(hipHostMalloc((void **)&e->h_tokens, sizeof(int) * max_batch, hipHostMallocDefault), "hipHostMalloc");
   b.hip(hipHostMalloc((void **)&e->h_next, sizeof(int) * max_batch, hipHostMallocDefault), "hipHostMalloc");
+  if (precise) {
+    int rc = create_precise(e, b, host_weights);
+    if (rc != GPTOSS_OK) {
+      destroy(e);
+      return rc;
+    }
+    *out = e;
+    return GPTOSS_OK;
+  }
 
   // staging: large enough for one expert's gate/up matrix, one qkv matrix and a slice of the
   // (un)embedding table
@@ -407,6 +539,14 @@ extern "C" int gptoss_engine_step(gptoss_engine *e, const int *host_tokens, int 
 
   memcpy(e->h_tokens, host_tokens, sizeof(int) * B);
   GPTOSS_HIP(hipMemcpyAsync(e->d_tokens, e->h_tokens, sizeof(int) * B, hipMemcpyHostToDevice, s));
+  if (e->flags & GPTOSS_ENGINE_PRECISE) {
+    STEP(precise_step(e, pos, B));
+    STEP(run_argmax(e->logits, e->d_next, B, V, s));
+    GPTOSS_HIP(hipMemcpyAsync(e->h_next, e->d_next, sizeof(int) * B, hipMemcpyDeviceToHost, s));
+    GPTOSS_HIP(hipStreamSynchronize(s));
+    memcpy(host_next, e->h_next, sizeof(int) * B);
+    return GPTOSS_OK;
+  }
   STEP(run_fill_int(e->d_lens, B, pos + 1, s));
   STEP(run_embedding(e->embedding, e->d_tokens, e->x, B, H, V, s));
   for (int l = 0; l < L; l++) {

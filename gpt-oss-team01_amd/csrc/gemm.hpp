@@ -32,6 +32,7 @@ int gemm_col_tiles(int N);  // column tiles of one workgroup's width
 // moe_route.hip
 int run_router(const void *t, const void *w_router, const float *b_router, float *logits, int B,
                int H, int E, int k, float *topk_w, int *topk_i, hipStream_t s);
+int run_topk_softmax(const float *logits, int B, int E, int k, float *topk_w, int *topk_i, hipStream_t s);
 int run_group(int B, int E, int k, float *topk_w, int *topk_i, int *expert_offsets,
               int *sorted_pair_ids, int *inv_perm, int *tiles, int rows_per_tile, hipStream_t s);
 

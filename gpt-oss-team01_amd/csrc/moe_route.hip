@@ -322,6 +322,19 @@ __global__ __launch_bounds__(SORT_THREADS) void group_sort_kernel(
 }
 
 
+// gating only: logits [B,E] -> top-k weights and ids
+int run_topk_softmax(const float *logits, int B, int E, int k, float *topk_w, int *topk_i, hipStream_t s) {
+  dim3 grid(cdiv(B * 32, 256)), block(256);
+  int nj = cdiv(E, 32);
+  TraceScope ts("topk_softmax", s);
+  if (nj <= 1) topk_softmax_kernel<1><<<grid, block, 0, s>>>(logits, B, E, k, topk_w, topk_i);
+  else if (nj <= 2) topk_softmax_kernel<2><<<grid, block, 0, s>>>(logits, B, E, k, topk_w, topk_i);
+  else if (nj <= 4) topk_softmax_kernel<4><<<grid, block, 0, s>>>(logits, B, E, k, topk_w, topk_i);
+  else topk_softmax_kernel<8><<<grid, block, 0, s>>>(logits, B, E, k, topk_w, topk_i);
+  GPTOSS_LAUNCH_CHECK("topk_softmax_kernel");
+  return GPTOSS_OK;
+}
+
 // logits (+ optional gating of the same tokens) in one launch
 int run_router(const void *t, const void *w_router, const float *b_router, float *logits, int B,
                int H, int E, int k, float *topk_w, int *topk_i, hipStream_t s) {
@@ -392,14 +405,8 @@ static int moe_route_impl(const float *logits, int B, int E, int k, float *topk_
   GPTOSS_REQUIRE(rows_per_tile == 0 || tiles, GPTOSS_ERR_NULL, "moe_route: tiles is NULL");
   hipStream_t s = (hipStream_t)stream;
   if (B > 0 && gate) {
-    dim3 grid(cdiv(B * 32, 256)), block(256);
-    int nj = cdiv(E, 32);
-    TraceScope ts("topk_softmax", s);
-    if (nj <= 1) topk_softmax_kernel<1><<<grid, block, 0, s>>>(logits, B, E, k, topk_w, topk_i);
-    else if (nj <= 2) topk_softmax_kernel<2><<<grid, block, 0, s>>>(logits, B, E, k, topk_w, topk_i);
-    else if (nj <= 4) topk_softmax_kernel<4><<<grid, block, 0, s>>>(logits, B, E, k, topk_w, topk_i);
-    else topk_softmax_kernel<8><<<grid, block, 0, s>>>(logits, B, E, k, topk_w, topk_i);
-    GPTOSS_LAUNCH_CHECK("topk_softmax_kernel");
+    int rc = run_topk_softmax(logits, B, E, k, topk_w, topk_i, s);
+    if (rc != GPTOSS_OK) return rc;
   }
   int nbits = 0;
   while ((1 << nbits) < E) nbits++;

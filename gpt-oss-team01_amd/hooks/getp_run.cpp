@@ -41,7 +41,10 @@ void warm_up(Transformer *transformer, Tokenizer *tokenizer) {
   if (max_batch < 1) max_batch = 1;
   // the reference caps the context at 1024 positions (getp-csrc/src/alloc.cpp:1047)
   g_gptoss_max_seq = cfg.seq_len < 1024 ? cfg.seq_len : 1024;
-  if (gptoss_engine_create(&cfg, weights, max_batch, g_gptoss_max_seq, 0, 0, &g_gptoss_engine) != GPTOSS_OK)
+  // GPTOSS_PRECISE=1: the CPU model's fp32/double arithmetic on the GPU (exact greedy ids, slow)
+  const char *precise = getenv("GPTOSS_PRECISE");
+  const int flags = (precise && atoi(precise) != 0) ? GPTOSS_ENGINE_PRECISE : 0;
+  if (gptoss_engine_create(&cfg, weights, max_batch, g_gptoss_max_seq, flags, 0, &g_gptoss_engine) != GPTOSS_OK)
     gptoss_die("engine_create");
 }
 

@@ -200,8 +200,10 @@ typedef struct gptoss_engine gptoss_engine;
 
 enum {
   GPTOSS_ENGINE_SYNTHETIC = 1, /* host_weights ignored: N(0,0.02) bf16 weights generated on device */
-  GPTOSS_ENGINE_PRECISE = 2    /* reserved: fp32-faithful activations instead of the reference GPU
-                                  path's bf16 staging; engine_create refuses it in this version */
+  GPTOSS_ENGINE_PRECISE = 2    /* the reference CPU model's arithmetic (run.cpp:501-717) instead of the
+                                  reference GPU path's bf16 staging: fp32 weights, activations and KV
+                                  cache, double-accumulated dot products.  Reproduces the CPU model's
+                                  greedy ids; slow, needs host_weights, 4x the weight memory */
 };
 
 /* Build device weights (bf16, packed) and run state for up to max_batch sequences of up to

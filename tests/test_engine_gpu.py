@@ -117,6 +117,46 @@ def test_generate_follows_getp_loop_semantics(ops, orc, tiny):
     assert (out[clear0, 0] == gold[clear0, 0]).all()
 
 
+def test_precise_engine_reproduces_the_golden_ids_exactly(ops, orc, tiny):
+    """GPTOSS_ENGINE_PRECISE runs the reference CPU model's arithmetic on the GPU (fp32 weights and
+    KV cache, double-accumulated dot products): free-running greedy generation must give exactly the
+    ids the reference's own CPU model produced (tests/golden/tiny_e2e.json, 8 x 32 ids), with the
+    getp loop's layout and count, and its logits must equal the CPU oracle's to fp32 rounding."""
+    fx, cfg, flat = tiny
+    prompts = np.asarray(fx["prompts"], np.int32)
+    gold = np.asarray(fx["expected_ids"], np.int32)
+    eng = ops.Engine(cfg, flat, max_batch=8, max_seq=fx["max_seq_len"], precise=True)
+    out, n = eng.generate(prompts, fx["max_seq_len"])
+    n_gen = gold.shape[1]
+    assert n == fx["n_generated"]
+    assert (out[:, fx["terminator_index"]] == -1).all()
+    assert np.array_equal(out[:, :n_gen], gold)
+    eng.close()
+    # teacher-forced logits against the fp32 oracle (bit-identical to the compiled reference)
+    B, T = 4, 40
+    seqs = np.concatenate([prompts[:B], gold[:B]], axis=1)[:, :T]
+    eng = ops.Engine(cfg, flat, max_batch=B, max_seq=64, precise=True)
+    cpu = [orc.Model(cfg, flat) for _ in range(B)]
+    worst = 0.0
+    for pos in range(T):
+        eng.step(seqs[:, pos], pos)
+        got = eng.last_logits(B)
+        for b in range(B):
+            want = cpu[b].forward(int(seqs[b, pos]), pos)
+            worst = max(worst, rel_errors(got[b], want)[0])
+    eng.close()
+    print("precise engine vs fp32 oracle, worst max-rel logit error:", worst)
+    assert worst <= 2e-5, worst
+
+
+def test_precise_engine_needs_host_weights(ops, tiny):
+    from conftest import load_pkg
+    lib = load_pkg("lib")
+    fx, cfg, flat = tiny
+    with pytest.raises(lib.GptossError):
+        ops.Engine(cfg, None, max_batch=2, max_seq=16, synthetic=True, precise=True)
+
+
 def test_engine_rejects_bad_arguments(ops, tiny):
     from conftest import load_pkg
     lib = load_pkg("lib")
