@@ -69,8 +69,10 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
   const int g = item % p.n_kv;
   const int rest = item / p.n_kv;
   const int b = rest % p.B;
-  const int chunk_id = rest / p.B;
-  if (chunk_id >= p.max_chunks) return;
+  // late chunks first: only long sequences have them, so the sparse part of the grid runs while
+  // the chip is still filling and the grid ends on chunk 0, which every sequence has
+  const int chunk_id = p.max_chunks - 1 - rest / p.B;
+  if (chunk_id < 0) return;
   const SeqRange r = seq_range(__builtin_amdgcn_readfirstlane(p.lens[b]), p.cap, p.window, p.chunk, p.max_len);
   if (chunk_id >= r.nchunks) return;
   // position held by slot s is s + pos_base, or cap less when that would lie beyond the last one
