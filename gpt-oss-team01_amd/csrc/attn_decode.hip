@@ -39,7 +39,8 @@ struct AttnParams {
 struct SeqRange {
   int s_begin, s_end;  // slot range to visit (s_begin is a multiple of 64)
   int t_lo, len;       // active positions are [t_lo, len)
-  int nchunks;
+  int nchunks;         // chunks the range is cut into (at most `chunk` slots each) ...
+  int chunk;           // ... of this many slots: the range split evenly, rounded up to 64
 };
 
 __device__ __forceinline__ SeqRange seq_range(int len, int cap, int window, int chunk, int max_len) {
@@ -55,52 +56,68 @@ __device__ __forceinline__ SeqRange seq_range(int len, int cap, int window, int 
     r.s_begin = 0;
     r.s_end = cap;
   }
-  r.nchunks = max(1, (r.s_end - r.s_begin + chunk - 1) / chunk);
+  const int span = r.s_end - r.s_begin;
+  r.nchunks = max(1, (span + chunk - 1) / chunk);
+  r.chunk = max(64, ((span + r.nchunks - 1) / r.nchunks + 63) & ~63);
   return r;
 }
 
 constexpr int ATT_MAX_BATCH = 2048;  // sequences per launch (four LDS ints each)
 
-// Persistent kernel.  Work item of a wave = (sequence, kv head, chunk of the sequence's slot range).
-// Every workgroup first builds the same item order in LDS from the sequence lengths: all full
-// chunks (sequence-major), then each sequence's last chunk, longest first in 64-slot buckets.  Wave
-// w takes items w, w + n_waves, ...: the rounds of this round-robin hold items of equal or
-// decreasing size, so static assignment balances like a longest-first list schedule without
-// atomics.  A wave's K/V double buffer keeps running across its items: while the last block of an
-// item is multiplied, the first block of the wave's next item is already on its way.
+// Persistent kernel.  Work item of a wave = (sequence, kv head, chunk of the sequence's slot range);
+// a sequence's range is cut into equal chunks, so item sizes only differ between sequences.
+// Every workgroup first builds the same item order in LDS from the sequence lengths: sequences
+// sorted by chunk size, largest first (counting sort over 32-slot size classes), each contributing
+// its chunks x kv heads.  Wave w takes item w of round 0, item n_waves-1-w of round 1, item w of
+// round 2, ...: a snake over a list sorted by size gives every wave nearly the same number of
+// slots without atomics.  A wave's K/V double buffer keeps running across its items: while the
+// last block of an item is multiplied, the first block of the wave's next item is already on its
+// way.
 template <int D>
 __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
   constexpr int KS = D / 32;   // k-steps of the score MFMA
   constexpr int DB = D / 16;   // 16-row blocks of O^T
   extern __shared__ int att_smem[];
   int *s_len = att_smem;             // [B]
-  int *s_pfull = att_smem + p.B;     // [B+1] exclusive prefix of full-chunk counts
-  int *s_plist = s_pfull + p.B + 1;  // [B] sequences ordered by the size of their last chunk
-  int *s_bkt = s_plist + p.B;        // [B] size bucket of each sequence's last chunk
+  int *s_pfull = att_smem + p.B;     // [B+1] exclusive prefix of the chunk counts, sorted order
+  int *s_plist = s_pfull + p.B + 1;  // [B] sequences ordered by chunk size, largest first
+  int *s_bkt = s_plist + p.B;        // [B] size class | chunk count << 4
   __shared__ int s_wsum[4];
-  __shared__ int s_bucket[8];
+  __shared__ int s_bucket[16];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
 
   // ---- item order --------------------------------------------------------------------------
-  if (threadIdx.x < 8) s_bucket[threadIdx.x] = 0;
+  if (threadIdx.x < 16) s_bucket[threadIdx.x] = 0;
   __syncthreads();
-  int running = 0;
-  for (int b0 = 0; b0 < p.B; b0 += 256) {
-    const int b = b0 + threadIdx.x;
-    int nfull = 0;
-    if (b < p.B) {
-      const int len = p.lens[b];
-      const SeqRange r = seq_range(len, p.cap, p.window, p.chunk, p.max_len);
-      nfull = r.nchunks - 1;
-      const int last_len = (r.s_end - r.s_begin) - nfull * p.chunk;
-      const int bucket = 7 - min(7, max(0, last_len - 1) >> 6);  // 0 = longest
-      s_len[b] = len;
-      s_bkt[b] = bucket;
-      atomicAdd(&s_bucket[bucket], 1);
+  for (int b = threadIdx.x; b < p.B; b += 256) {
+    const int len = p.lens[b];
+    const SeqRange r = seq_range(len, p.cap, p.window, p.chunk, p.max_len);
+    const int bucket = 15 - min(15, (r.chunk - 1) >> 5);  // 0 = largest chunks
+    s_len[b] = len;
+    s_bkt[b] = bucket | (r.nchunks << 4);
+    atomicAdd(&s_bucket[bucket], 1);
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int acc = 0;
+    for (int k = 0; k < 16; k++) {  // bucket counts -> bucket start cursors
+      int c = s_bucket[k];
+      s_bucket[k] = acc;
+      acc += c;
     }
-    // exclusive scan of nfull over this group of 256 sequences
-    int inc = nfull;
+  }
+  __syncthreads();
+  // scatter the sequences into their buckets; the order inside a bucket does not matter (every
+  // item's result is independent of the item order)
+  for (int b = threadIdx.x; b < p.B; b += 256) s_plist[atomicAdd(&s_bucket[s_bkt[b] & 15], 1)] = b;
+  __syncthreads();
+  // exclusive prefix of the chunk counts in sorted order
+  int running = 0;
+  for (int r0 = 0; r0 < p.B; r0 += 256) {
+    const int rk = r0 + threadIdx.x;
+    const int cnt = (rk < p.B) ? (s_bkt[s_plist[rk]] >> 4) : 0;
+    int inc = cnt;
 #pragma unroll
     for (int d = 1; d < 64; d <<= 1) {
       int o = __shfl_up(inc, d, 64);
@@ -110,27 +127,17 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
     __syncthreads();
     int base = running;
     for (int w = 0; w < wave; w++) base += s_wsum[w];
-    if (b < p.B) s_pfull[b] = base + inc - nfull;
+    if (rk < p.B) s_pfull[rk] = base + inc - cnt;
     running += s_wsum[0] + s_wsum[1] + s_wsum[2] + s_wsum[3];
     __syncthreads();
   }
-  if (threadIdx.x == 0) {
-    s_pfull[p.B] = running;
-    int acc = 0;
-    for (int k = 0; k < 8; k++) {  // bucket counts -> bucket start cursors
-      int c = s_bucket[k];
-      s_bucket[k] = acc;
-      acc += c;
-    }
-  }
+  if (threadIdx.x == 0) s_pfull[p.B] = running;
   __syncthreads();
-  // scatter the sequences into their buckets; the order inside a bucket does not matter (every
-  // item's result is independent of the item order)
-  for (int b = threadIdx.x; b < p.B; b += 256) s_plist[atomicAdd(&s_bucket[s_bkt[b]], 1)] = b;
-  __syncthreads();
-  const int total_full = s_pfull[p.B];
-  const int n_items = (total_full + p.B) * p.n_kv;
-  const int stride = gridDim.x * 4;
+  const int n_items = s_pfull[p.B] * p.n_kv;
+  const int n_waves = gridDim.x * 4;
+  const int wave_id = blockIdx.x * 4 + wave;
+  // item of this wave in round k of the snake
+  auto item_index = [&](int k) { return k * n_waves + ((k & 1) ? n_waves - 1 - wave_id : wave_id); };
 
   const int n = lane & 15, c = lane >> 4;
   const int G = p.G;
@@ -146,34 +153,29 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
     Item it;
     const int pair = i / p.n_kv;
     it.g = i - pair * p.n_kv;
-    int b, chunk_id = -1;
-    if (pair < total_full) {  // largest b with pfull[b] <= pair
-      int lo = 0, hi = p.B;
-      while (hi - lo > 1) {
-        const int mid = (lo + hi) >> 1;
-        if (s_pfull[mid] <= pair) lo = mid;
-        else hi = mid;
-      }
-      b = lo;
-      chunk_id = pair - s_pfull[b];
-    } else {
-      b = s_plist[pair - total_full];
+    int lo = 0, hi = p.B;  // largest rank with pfull[rank] <= pair
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if (s_pfull[mid] <= pair) lo = mid;
+      else hi = mid;
     }
+    int b = s_plist[lo];
+    int chunk_id = pair - s_pfull[lo];
     b = __builtin_amdgcn_readfirstlane(b);
     const SeqRange r = seq_range(__builtin_amdgcn_readfirstlane(s_len[b]), p.cap, p.window, p.chunk, p.max_len);
-    if (chunk_id < 0) chunk_id = r.nchunks - 1;
     it.b = b;
     it.chunk_id = __builtin_amdgcn_readfirstlane(chunk_id);
     it.nchunks = r.nchunks;
     it.len = r.len;
     it.t_lo = r.t_lo;
-    it.c0 = r.s_begin + it.chunk_id * p.chunk;
-    it.c1 = min(r.s_end, it.c0 + p.chunk);
+    it.c0 = r.s_begin + it.chunk_id * r.chunk;
+    it.c1 = min(r.s_end, it.c0 + r.chunk);
     it.has = it.c1 > it.c0;
     return it;
   };
 
-  int i = blockIdx.x * 4 + wave;  // wave-uniform: everything derived from it stays scalar
+  int round = 0;
+  int i = item_index(0);  // wave-uniform: everything derived from it stays scalar
   if (i >= n_items) return;
   Item cur = decode(i);
 
@@ -199,7 +201,7 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
   bool have_first = false;  // the first block of `cur` is already in (or on its way to) buffer 0
 
   while (true) {
-    const int i_next = i + stride;
+    const int i_next = item_index(round + 1);
     const bool more = i_next < n_items;
     const Item nxt = more ? decode(i_next) : cur;
     const bool nxt_has = more && nxt.has;
@@ -402,6 +404,7 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
     }
     cur = nxt;
     i = i_next;
+    round++;
   }
 }
 
