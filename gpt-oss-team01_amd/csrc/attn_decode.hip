@@ -17,6 +17,7 @@
 #include <type_traits>
 
 #include "common.hpp"
+#include "glue.hpp"
 
 namespace gptoss {
 
@@ -32,6 +33,7 @@ struct AttnParams {
   bf16_t *out;         // [B, n_q, D]
   float *part_o;       // [B, max_chunks, n_q, D]
   float *part_ml;      // [B, max_chunks, n_q, 2]
+  int *ticket;         // work counter (zero on entry) for the dynamically dealt tail, or nullptr
   int B, n_q, n_kv, G, cap, window, chunk, max_chunks, max_len;
   float scale_log2e;   // log2(e) / sqrt(D)
 };
@@ -62,6 +64,8 @@ __device__ __forceinline__ SeqRange seq_range(int len, int cap, int window, int 
   return r;
 }
 
+constexpr int ATT_THREADS = 512;     // one workgroup of 8 waves per CU (two waves per SIMD)
+constexpr int ATT_WAVES = ATT_THREADS / 64;
 constexpr int ATT_MAX_BATCH = 2048;  // sequences per launch (four LDS ints each)
 
 // Persistent kernel.  Work item of a wave = (sequence, kv head, chunk of the sequence's slot range);
@@ -70,11 +74,14 @@ constexpr int ATT_MAX_BATCH = 2048;  // sequences per launch (four LDS ints each
 // sorted by chunk size, largest first (counting sort over 32-slot size classes), each contributing
 // its chunks x kv heads.  Wave w takes item w of round 0, item n_waves-1-w of round 1, item w of
 // round 2, ...: a snake over a list sorted by size gives every wave nearly the same number of
-// slots without atomics.  A wave's K/V double buffer keeps running across its items: while the
+// slots.  Waves do not stream equally fast (the second wave of a SIMD gets less than the first,
+// and CUs differ by some 10 %), so when there are at least three rounds the last full round and
+// the remainder - the smallest items - are handed out through a counter instead, one atomic per
+// item, requested a whole item before its result is needed.  A wave's K/V double buffer keeps running across its items: while the
 // last block of an item is multiplied, the first block of the wave's next item is already on its
 // way.
 template <int D>
-__global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
+__global__ __launch_bounds__(ATT_THREADS, 1) void attn_decode_kernel(AttnParams p) {
   constexpr int KS = D / 32;   // k-steps of the score MFMA
   constexpr int DB = D / 16;   // 16-row blocks of O^T
   extern __shared__ int att_smem[];
@@ -82,7 +89,7 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
   int *s_pfull = att_smem + p.B;     // [B+1] exclusive prefix of the chunk counts, sorted order
   int *s_plist = s_pfull + p.B + 1;  // [B] sequences ordered by chunk size, largest first
   int *s_bkt = s_plist + p.B;        // [B] size class | chunk count << 4
-  __shared__ int s_wsum[4];
+  __shared__ int s_wsum[ATT_WAVES];
   __shared__ int s_bucket[16];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -90,7 +97,7 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
   // ---- item order --------------------------------------------------------------------------
   if (threadIdx.x < 16) s_bucket[threadIdx.x] = 0;
   __syncthreads();
-  for (int b = threadIdx.x; b < p.B; b += 256) {
+  for (int b = threadIdx.x; b < p.B; b += ATT_THREADS) {
     const int len = p.lens[b];
     const SeqRange r = seq_range(len, p.cap, p.window, p.chunk, p.max_len);
     const int bucket = 15 - min(15, (r.chunk - 1) >> 5);  // 0 = largest chunks
@@ -110,11 +117,11 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
   __syncthreads();
   // scatter the sequences into their buckets; the order inside a bucket does not matter (every
   // item's result is independent of the item order)
-  for (int b = threadIdx.x; b < p.B; b += 256) s_plist[atomicAdd(&s_bucket[s_bkt[b] & 15], 1)] = b;
+  for (int b = threadIdx.x; b < p.B; b += ATT_THREADS) s_plist[atomicAdd(&s_bucket[s_bkt[b] & 15], 1)] = b;
   __syncthreads();
   // exclusive prefix of the chunk counts in sorted order
   int running = 0;
-  for (int r0 = 0; r0 < p.B; r0 += 256) {
+  for (int r0 = 0; r0 < p.B; r0 += ATT_THREADS) {
     const int rk = r0 + threadIdx.x;
     const int cnt = (rk < p.B) ? (s_bkt[s_plist[rk]] >> 4) : 0;
     int inc = cnt;
@@ -128,17 +135,20 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
     int base = running;
     for (int w = 0; w < wave; w++) base += s_wsum[w];
     if (rk < p.B) s_pfull[rk] = base + inc - cnt;
-    running += s_wsum[0] + s_wsum[1] + s_wsum[2] + s_wsum[3];
+    for (int w = 0; w < ATT_WAVES; w++) running += s_wsum[w];
     __syncthreads();
   }
   if (threadIdx.x == 0) s_pfull[p.B] = running;
   __syncthreads();
   const int n_items = s_pfull[p.B] * p.n_kv;
-  const int n_waves = gridDim.x * 4;
-  const int wave_id = blockIdx.x * 4 + wave;
+  const int n_waves = gridDim.x * ATT_WAVES;
+  const int wave_id = blockIdx.x * ATT_WAVES + wave;
   // item of this wave in round k of the snake
   auto item_index = [&](int k) { return k * n_waves + ((k & 1) ? n_waves - 1 - wave_id : wave_id); };
-
+  const int full_rounds = n_items / n_waves;
+  const bool use_tickets = p.ticket != nullptr && full_rounds >= 3;
+  const int static_rounds = use_tickets ? full_rounds - 1 : 0x3fffffff;
+  const int pool_base = use_tickets ? static_rounds * n_waves : 0;
   const int n = lane & 15, c = lane >> 4;
   const int G = p.G;
   // lane's K bytes for slot block `blk`: slot blk + tb*16 + n, d chunk c*KS*8 .. +KS*8
@@ -201,10 +211,22 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
   bool have_first = false;  // the first block of `cur` is already in (or on its way to) buffer 0
 
   while (true) {
-    const int i_next = item_index(round + 1);
-    const bool more = i_next < n_items;
-    const Item nxt = more ? decode(i_next) : cur;
-    const bool nxt_has = more && nxt.has;
+    // the wave's next item: by position while the static rounds last, then by ticket.  The ticket
+    // is requested now and only read when the last block of this item is reached.
+    const bool ticket_next = round + 1 >= static_rounds;
+    int ticket = 0;
+    if (ticket_next && lane == 0) ticket = atomicAdd(p.ticket, 1);
+    int i_next = 0;
+    bool more = false, nxt_has = false, resolved = false;
+    Item nxt = cur;
+    auto resolve_next = [&]() {
+      if (resolved) return;
+      resolved = true;
+      i_next = ticket_next ? pool_base + __builtin_amdgcn_readfirstlane(ticket) : item_index(round + 1);
+      more = i_next < n_items;
+      if (more) nxt = decode(i_next);
+      nxt_has = more && nxt.has;
+    };
     if (cur.has && !have_first) load_kv(cur, cur.c0, R0{});
     have_first = false;
 
@@ -334,9 +356,13 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
     // of the wave's next item, else (nothing left to fetch) this item's last block again
     const int last_blk = max(cur.c0, ((c1 - 1) & ~(ATT_BLOCK - 1)));
     auto prefetch = [&](int blk, auto buf) {
-      if (blk + ATT_BLOCK < c1) load_kv(cur, blk + ATT_BLOCK, buf);
-      else if (nxt_has) load_kv(nxt, nxt.c0, buf);
-      else load_kv(cur, last_blk, buf);
+      if (blk + ATT_BLOCK < c1) {
+        load_kv(cur, blk + ATT_BLOCK, buf);
+      } else {
+        resolve_next();
+        if (nxt_has) load_kv(nxt, nxt.c0, buf);
+        else load_kv(cur, last_blk, buf);
+      }
     };
 
     int parity = 0;  // buffer that received the last prefetch
@@ -360,6 +386,7 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
       }
       have_first = nxt_has;
     }
+    resolve_next();
 
     // ---- per-head totals: sum the partial denominators of the 4 lanes that share a head --------
     l_run += __shfl_xor(l_run, 16, 64);
@@ -492,6 +519,7 @@ static int attn_chunk_tokens(int span) { return span > 1024 ? 512 : 256; }
 struct AttnPlan {
   int chunk, max_chunks;
   size_t part_o_bytes, part_ml_bytes;
+  static constexpr size_t ticket_bytes = 256;  // one counter per slice of ATT_MAX_BATCH sequences
 };
 
 static AttnPlan attn_plan(int B, int n_q, int D, int max_len) {
@@ -538,7 +566,7 @@ extern "C" size_t gptoss_attn_workspace_bytes(int B, int n_q, int n_kv, int head
   // sized for the smallest chunk length so that any window/capacity combination fits
   int max_chunks = (max_len + ATT_BLOCK - 1 + 255) / 256;
   return align_up((size_t)B * max_chunks * n_q * head_dim * sizeof(float), 256) +
-         align_up((size_t)B * max_chunks * n_q * 2 * sizeof(float), 256);
+         align_up((size_t)B * max_chunks * n_q * 2 * sizeof(float), 256) + AttnPlan::ticket_bytes;
 }
 
 extern "C" int gptoss_attn_decode(const float *q, const void *k_cache, const void *v_cache,
@@ -562,9 +590,9 @@ extern "C" int gptoss_attn_decode(const float *q, const void *k_cache, const voi
                                   : ((window > 0 && window < max_len) ? window : max_len);
   AttnPlan pl = attn_plan(B, n_q, head_dim, span);
   GPTOSS_REQUIRE(workspace && aligned(workspace, 256) &&
-                     workspace_bytes >= pl.part_o_bytes + pl.part_ml_bytes,
+                     workspace_bytes >= pl.part_o_bytes + pl.part_ml_bytes + pl.ticket_bytes,
                  GPTOSS_ERR_WORKSPACE, "attn_decode: workspace missing, misaligned or smaller than %zu bytes",
-                 pl.part_o_bytes + pl.part_ml_bytes);
+                 pl.part_o_bytes + pl.part_ml_bytes + pl.ticket_bytes);
   AttnParams p;
   p.q = q;
   p.kc = (const bf16_t *)k_cache;
@@ -574,6 +602,7 @@ extern "C" int gptoss_attn_decode(const float *q, const void *k_cache, const voi
   p.out = (bf16_t *)out;
   p.part_o = (float *)workspace;
   p.part_ml = (float *)((unsigned char *)workspace + pl.part_o_bytes);
+  p.ticket = (int *)((unsigned char *)workspace + pl.part_o_bytes + pl.part_ml_bytes);
   p.B = B;
   p.n_q = n_q;
   p.n_kv = n_kv;
@@ -585,12 +614,33 @@ extern "C" int gptoss_attn_decode(const float *q, const void *k_cache, const voi
   p.max_len = max_len;
   p.scale_log2e = 1.4426950408889634f / sqrtf((float)head_dim);
   hipStream_t s = (hipStream_t)stream;
-  // persistent grid: two workgroups of four waves per CU, fewer when there is less work; batches
+  // persistent grid: one workgroup of eight waves per CU, fewer when there is less work; batches
   // beyond ATT_MAX_BATCH sequences (the kernel keeps four ints per sequence in LDS) are sliced
+  GPTOSS_REQUIRE(B <= ATT_MAX_BATCH * (int)(AttnPlan::ticket_bytes / sizeof(int)), GPTOSS_ERR_DIM,
+                 "attn_decode: at most %d sequences per call", ATT_MAX_BATCH * (int)(AttnPlan::ticket_bytes / sizeof(int)));
+  // tickets are only used for long contexts (512-slot chunks: an item then lasts tens of
+  // microseconds, against which one atomic is nothing) when a slice can have three or more rounds
+  // of items; the counters start at zero (a fill kernel rather than a memset, so that the call can
+  // be captured in a graph)
+  bool any_tickets = false;
+  for (int b0 = 0; b0 < B; b0 += ATT_MAX_BATCH) {
+    const int nb = (B - b0 < ATT_MAX_BATCH) ? B - b0 : ATT_MAX_BATCH;
+    const long long items = (long long)nb * n_kv * pl.max_chunks;
+    long long grid = (items + ATT_WAVES - 1) / ATT_WAVES;
+    if (grid > 256) grid = 256;
+    if (pl.chunk >= 512 && items / (grid * ATT_WAVES) >= 3) any_tickets = true;
+  }
+  if (any_tickets) {
+    int rc = run_fill_int(p.ticket, (int)(AttnPlan::ticket_bytes / sizeof(int)), 0, s);
+    if (rc != GPTOSS_OK) return rc;
+  } else {
+    p.ticket = nullptr;
+  }
   {
     TraceScope ts("attn_decode", s);
     for (int b0 = 0; b0 < B; b0 += ATT_MAX_BATCH) {
       AttnParams ps = p;
+      if (p.ticket) ps.ticket = p.ticket + b0 / ATT_MAX_BATCH;
       ps.B = (B - b0 < ATT_MAX_BATCH) ? B - b0 : ATT_MAX_BATCH;
       ps.q = p.q + (size_t)b0 * n_q * head_dim;
       ps.kc = p.kc + (size_t)b0 * n_kv * capacity * head_dim;
@@ -600,11 +650,11 @@ extern "C" int gptoss_attn_decode(const float *q, const void *k_cache, const voi
       ps.part_o = p.part_o + (size_t)b0 * pl.max_chunks * n_q * head_dim;
       ps.part_ml = p.part_ml + (size_t)b0 * pl.max_chunks * n_q * 2;
       long long items = (long long)ps.B * n_kv * pl.max_chunks;
-      int grid = (int)((items + 3) / 4);
-      if (grid > 512) grid = 512;
+      int grid = (int)((items + ATT_WAVES - 1) / ATT_WAVES);
+      if (grid > 256) grid = 256;
       const size_t smem = sizeof(int) * (4 * (size_t)ps.B + 1);
-      if (head_dim == 64) attn_decode_kernel<64><<<grid, 256, smem, s>>>(ps);
-      else attn_decode_kernel<32><<<grid, 256, smem, s>>>(ps);
+      if (head_dim == 64) attn_decode_kernel<64><<<grid, ATT_THREADS, smem, s>>>(ps);
+      else attn_decode_kernel<32><<<grid, ATT_THREADS, smem, s>>>(ps);
     }
   }
   GPTOSS_LAUNCH_CHECK("attn_decode_kernel");
