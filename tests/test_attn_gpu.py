@@ -125,3 +125,39 @@ def test_attn_bad_arguments(ops):
     assert rc == 2 and "head_dim" in lib.last_error()
     rc = L.gptoss_attn_decode(None, None, None, None, None, None, 1, 8, 2, 64, 64, 0, 10, None, 0, None)
     assert rc == 1
+
+
+def test_attn_many_long_sequences_static_and_ticket_rounds(ops, orc):
+    """Enough long sequences that every persistent wave works through several rounds of items and
+    the tail is handed out through the work counter (>= 3 rounds of 512-slot chunks); lengths from
+    0 to the full 4096, the result twice in a row from the same workspace."""
+    B, n_q, n_kv, D, S = 160, 16, 8, 64, 4096
+    rng = np.random.default_rng(42)
+    lens = rng.integers(1, S + 1, size=B).astype(np.int32)
+    lens[:4] = [0, 1, S, 513]
+    q, K, V, sinks = _mk(B, S, n_q, n_kv, D, seed=3)
+    cache = ops.KVCache(B, n_kv, D, S)
+    cache.k.view(torch.int16).fill_(0x7FC1)
+    cache.v.view(torch.int16).fill_(0x7FC1)
+    cache.write(K.cuda(), V.cuda(), 0)
+    attn = ops.AttnDecode(B, n_q, n_kv, D, S)
+    lens_d = torch.as_tensor(lens).cuda()
+    a = attn.forward(q.cuda(), cache, lens_d, sinks.cuda(), window=0).float().cpu().numpy()
+    b = attn.forward(q.cuda(), cache, lens_d, sinks.cuda(), window=0).float().cpu().numpy()
+    assert np.array_equal(a, b)                       # the counter is reset per call; deterministic
+    want = orc.attn_decode(q.numpy(), K.float().numpy(), V.float().numpy(), lens, sinks.numpy(), 0)
+    assert np.isfinite(a).all()
+    mx, mean = rel_errors(a, want)
+    assert mx <= TOL_MAX and mean <= TOL_MEAN, (mx, mean)
+
+
+def test_attn_batch_larger_than_one_launch_slice(ops, orc):
+    """More sequences than one launch keeps in LDS (2048): the call is sliced internally."""
+    B, n_q, n_kv, D, S = 2100, 2, 1, 32, 64
+    rng = np.random.default_rng(7)
+    lens = rng.integers(1, S + 1, size=B).astype(np.int32)
+    q, K, V, sinks = _mk(B, S, n_q, n_kv, D, seed=9)
+    got = _run(ops, q, K, V, lens, sinks, 0)
+    want = orc.attn_decode(q.numpy(), K.float().numpy(), V.float().numpy(), lens, sinks.numpy(), 0)
+    mx, mean = rel_errors(got, want)
+    assert mx <= TOL_MAX and mean <= TOL_MEAN, (mx, mean)
