@@ -291,7 +291,8 @@ def bench_e2e(ops, torch, n_req=1024, n_prompt=128, n_decode=256):
     synth = importlib.import_module("gpt-oss-team01_amd.synth")
     cfg = synth.gptoss20b_config(max_seq_len=n_prompt + n_decode)
     t0 = time.perf_counter()
-    eng = ops.Engine(cfg, None, max_batch=n_req, max_seq=n_prompt + n_decode, synthetic=True, seed=1)
+    eng = ops.Engine(cfg, None, max_batch=n_req, max_seq=n_prompt + n_decode, synthetic=True, seed=1,
+                     keep_logits=False)
     t_create = time.perf_counter() - t0
     rng = np.random.default_rng(3)
     prompts = rng.integers(0, cfg.vocab_size, size=(n_req, n_prompt), dtype=np.int32)

@@ -54,7 +54,9 @@ struct gptoss_engine {
   // run state
   int *d_tokens, *d_next, *d_lens;
   int *h_tokens, *h_next;  // pinned
-  float *x, *qkv, *q, *tb2, *logits;
+  float *x, *qkv, *q, *tb2, *logits;  // logits == nullptr unless GPTOSS_ENGINE_LOGITS
+  float *amax_val;                     // [B, column tiles of the classifier]: fused arg-max partials
+  int *amax_idx;
   bf16_t *t, *attn_out;
   void *moe_ws, *attn_ws;
   size_t moe_ws_bytes, attn_ws_bytes;
@@ -187,8 +189,10 @@ void rope_tables(const gptoss_config &c, int n_pos, std::vector<float> &cs, std:
 }
 
 int dense_gemm(const bf16_t *A, const bf16_t *W, const float *bias, void *out, int epi, int B, int N,
-               int K, hipStream_t s) {
+               int K, hipStream_t s, float *amax_val = nullptr, int *amax_idx = nullptr) {
   GemmParams g{};
+  g.amax_val = amax_val;
+  g.amax_idx = amax_idx;
   g.A = A;
   g.W = W;
   g.bias = bias;
@@ -505,7 +509,15 @@ extern "C" int gptoss_engine_create(const gptoss_config *cfg, const float *host_
   e->q = b.alloc<float>((size_t)B * nq * D);
   e->attn_out = b.alloc<bf16_t>((size_t)B * nq * D);
   e->tb2 = b.alloc<float>((size_t)B * H);
-  e->logits = b.alloc<float>((size_t)B * V);
+  e->logits = nullptr;
+  e->amax_val = nullptr;
+  e->amax_idx = nullptr;
+  if (flags & GPTOSS_ENGINE_LOGITS) {
+    e->logits = b.alloc<float>((size_t)B * V);
+  } else {
+    e->amax_val = b.alloc<float>((size_t)B * gemm_col_tiles(V));
+    e->amax_idx = b.alloc<int>((size_t)B * gemm_col_tiles(V));
+  }
   e->moe_ws_bytes = gptoss_moe_workspace_bytes(B, E, k, H, I);
   e->moe_ws = b.alloc<unsigned char>(e->moe_ws_bytes);
   e->attn_ws_bytes = std::max<size_t>(256, gptoss_attn_workspace_bytes(B, nq, nkv, D, max_seq));
@@ -578,8 +590,15 @@ extern "C" int gptoss_engine_step(gptoss_engine *e, const int *host_tokens, int 
     const float *nw = (l + 1 < L) ? e->layers[l + 1].attn_norm : e->final_norm;
     STEP(run_rmsnorm(e->x, nullptr, nw, e->t, nullptr, B, H, s));
   }
-  STEP(dense_gemm(e->t, e->unembedding, nullptr, e->logits, EPI_F32, B, V, H, s));
-  STEP(run_argmax(e->logits, e->d_next, B, V, s));
+  if (e->logits) {
+    STEP(dense_gemm(e->t, e->unembedding, nullptr, e->logits, EPI_F32, B, V, H, s));
+    STEP(run_argmax(e->logits, e->d_next, B, V, s));
+  } else {
+    // the classifier keeps only (max, column) per row and column tile; a small second stage picks
+    // the row's arg-max (lowest column among equal maxima, run.cpp:739-750)
+    STEP(dense_gemm(e->t, e->unembedding, nullptr, nullptr, EPI_ARGMAX, B, V, H, s, e->amax_val, e->amax_idx));
+    STEP(run_argmax_tiles(e->amax_val, e->amax_idx, e->d_next, B, gemm_col_tiles(V), s));
+  }
   GPTOSS_HIP(hipMemcpyAsync(e->h_next, e->d_next, sizeof(int) * B, hipMemcpyDeviceToHost, s));
   GPTOSS_HIP(hipStreamSynchronize(s));
   memcpy(host_next, e->h_next, sizeof(int) * B);

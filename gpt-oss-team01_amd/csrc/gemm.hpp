@@ -4,7 +4,7 @@
 
 namespace gptoss {
 
-enum { EPI_F32 = 0, EPI_SWIGLU = 1, EPI_BF16 = 2 };
+enum { EPI_F32 = 0, EPI_SWIGLU = 1, EPI_BF16 = 2, EPI_ARGMAX = 3 };
 
 struct GemmParams {
   const bf16_t *A;     // activations, row-major [*, K]
@@ -14,6 +14,8 @@ struct GemmParams {
   int w_mxfp4;         // W holds gptoss_pack_mxfp4 output
   const float *bias;   // [n_mat, N] or nullptr
   void *out;           // EPI_F32: float [*, N]; EPI_SWIGLU: bf16 [*, N/2]; EPI_BF16: bf16 [*, N]
+  float *amax_val;     // EPI_ARGMAX (dense only): per (row, column tile) the largest value ...
+  int *amax_idx;       // ... and the lowest column that holds it, [rows, n_col_tiles]
   const int *tiles;    // {n_tiles, (mat,row0,rows)*} or nullptr for a dense problem
   int dense_rows;      // rows of the dense problem when tiles == nullptr
   int N, K;

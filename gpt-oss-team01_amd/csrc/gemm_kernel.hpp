@@ -263,6 +263,59 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, bf16_t *lds, int 
   for (int s = 0; s < padded; s += NRING)
     static_for<0, NRING>([&](auto r) { body(s + (int)decltype(r)::value, r); });
 
+  if (EPI == EPI_ARGMAX) {
+    // Row-wise arg-max of this workgroup's 256 columns without writing the products: every lane
+    // reduces its 16 channels (ascending, strict >, so the lowest column wins a tie), the two
+    // half-waves are merged, the 8 waves meet in LDS (free since the last barrier) and one thread
+    // per row writes the tile's (value, column) pair.
+    float *rv = reinterpret_cast<float *>(lds);
+    int *ri = reinterpret_cast<int *>(lds) + GEMM_WAVES * MBMAX * 32;
+    const int tok = lane & 31, h4 = (lane >> 5) * 4;
+#pragma unroll
+    for (int i = 0; i < MB; i++) {
+      float bv = -INFINITY;
+      int bi = 0x7fffffff;
+      if (wave_active) {
+#pragma unroll
+        for (int g = 0; g < 4; g++)
+#pragma unroll
+          for (int q = 0; q < 4; q++) {
+            const int col = n0 + g * 8 + h4 + q;
+            const float v = acc[i][g * 4 + q] + (p.bias ? p.bias[(size_t)mat * N + col] : 0.f);
+            if (v > bv) {
+              bv = v;
+              bi = col;
+            }
+          }
+      }
+      const float ov = __shfl_xor(bv, 32, 64);
+      const int oi = __shfl_xor(bi, 32, 64);
+      if (ov > bv || (ov == bv && oi < bi)) {
+        bv = ov;
+        bi = oi;
+      }
+      if (lane < 32) {
+        rv[wave * (MBMAX * 32) + i * 32 + tok] = bv;
+        ri[wave * (MBMAX * 32) + i * 32 + tok] = bi;
+      }
+    }
+    __syncthreads();
+    if (tid < MB * 32 && tid < rows) {
+      float bv = rv[tid];
+      int bi = ri[tid];
+#pragma unroll
+      for (int w = 1; w < GEMM_WAVES; w++) {
+        const float v = rv[w * (MBMAX * 32) + tid];
+        if (v > bv) {  // later waves hold higher columns: ties keep the earlier one
+          bv = v;
+          bi = ri[w * (MBMAX * 32) + tid];
+        }
+      }
+      p.amax_val[(size_t)(row0 + tid) * p.n_col_tiles + ct] = bv;
+      p.amax_idx[(size_t)(row0 + tid) * p.n_col_tiles + ct] = bi;
+    }
+    return;
+  }
   if (!wave_active) return;
 
   // ---- epilogue ------------------------------------------------------------------------------
@@ -445,8 +498,9 @@ int launch_gemm(const GemmParams &p, int max_tiles, hipStream_t s) {
   if (grid > resident) grid = resident;
   if (grid == 0) return GPTOSS_OK;
   {
-    TraceScope ts(FP4 ? (GATHER ? "gemm1_gather_swiglu_mxfp4" : "gemm_f32_mxfp4")
-                      : (GATHER ? "gemm1_gather_swiglu" : "gemm_f32"), s);
+    TraceScope ts(EPI == EPI_ARGMAX ? "gemm_argmax"
+                  : FP4 ? (GATHER ? "gemm1_gather_swiglu_mxfp4" : "gemm_f32_mxfp4")
+                        : (GATHER ? "gemm1_gather_swiglu" : "gemm_f32"), s);
     hipLaunchKernelGGL(kern, dim3(grid), dim3(GEMM_THREADS), smem, s, p);
   }
   GPTOSS_LAUNCH_CHECK("grouped_gemm_kernel");
@@ -463,6 +517,11 @@ int launch_gemm(const GemmParams &p, int max_tiles, hipStream_t s) {
   template int launch_gemm<2, false, EPI_F32, FP4V>(const GemmParams &, int, hipStream_t);     \
   template int launch_gemm<3, false, EPI_F32, FP4V>(const GemmParams &, int, hipStream_t);     \
   template int launch_gemm<4, false, EPI_F32, FP4V>(const GemmParams &, int, hipStream_t);     \
-  template int launch_gemm<5, false, EPI_F32, FP4V>(const GemmParams &, int, hipStream_t);
+  template int launch_gemm<5, false, EPI_F32, FP4V>(const GemmParams &, int, hipStream_t);     \
+  template int launch_gemm<1, false, EPI_ARGMAX, FP4V>(const GemmParams &, int, hipStream_t);  \
+  template int launch_gemm<2, false, EPI_ARGMAX, FP4V>(const GemmParams &, int, hipStream_t);  \
+  template int launch_gemm<3, false, EPI_ARGMAX, FP4V>(const GemmParams &, int, hipStream_t);  \
+  template int launch_gemm<4, false, EPI_ARGMAX, FP4V>(const GemmParams &, int, hipStream_t);  \
+  template int launch_gemm<5, false, EPI_ARGMAX, FP4V>(const GemmParams &, int, hipStream_t);
 
 }  // namespace gptoss

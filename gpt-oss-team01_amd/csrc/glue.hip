@@ -201,6 +201,54 @@ int run_rope_store(const float *qkv, float *q_out, bf16_t *kc, bf16_t *vc, const
   return GPTOSS_OK;
 }
 
+// ids[b] = column of the largest per-tile maximum, lowest column among equal ones: the second
+// stage of the arg-max that the classifier GEMM's epilogue starts.
+__global__ __launch_bounds__(256) void argmax_tiles_kernel(const float *__restrict__ val,
+                                                           const int *__restrict__ idx,
+                                                           int *__restrict__ ids, int n_tiles) {
+  __shared__ float sv[4];
+  __shared__ int si[4];
+  const int b = blockIdx.x;
+  float bv = -INFINITY;
+  int bi = 0x7fffffff;
+  for (int t = threadIdx.x; t < n_tiles; t += 256) {
+    const float v = val[(size_t)b * n_tiles + t];
+    const int i = idx[(size_t)b * n_tiles + t];
+    if (v > bv || (v == bv && i < bi)) {
+      bv = v;
+      bi = i;
+    }
+  }
+  for (int m = 32; m >= 1; m >>= 1) {
+    const float ov = __shfl_xor(bv, m, 64);
+    const int oi = __shfl_xor(bi, m, 64);
+    if (ov > bv || (ov == bv && oi < bi)) {
+      bv = ov;
+      bi = oi;
+    }
+  }
+  if ((threadIdx.x & 63) == 0) {
+    sv[threadIdx.x >> 6] = bv;
+    si[threadIdx.x >> 6] = bi;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < 4; w++)
+      if (sv[w] > bv || (sv[w] == bv && si[w] < bi)) {
+        bv = sv[w];
+        bi = si[w];
+      }
+    ids[b] = bi == 0x7fffffff ? 0 : bi;
+  }
+}
+
+int run_argmax_tiles(const float *val, const int *idx, int *ids, int B, int n_tiles, hipStream_t s) {
+  TraceScope ts("argmax_tiles", s);
+  argmax_tiles_kernel<<<B, 256, 0, s>>>(val, idx, ids, n_tiles);
+  GPTOSS_LAUNCH_CHECK("argmax_tiles_kernel");
+  return GPTOSS_OK;
+}
+
 int run_argmax(const float *logits, int *ids, int B, int V, hipStream_t s) {
   TraceScope ts("argmax", s);
   argmax_kernel<<<B, 1024, 0, s>>>(logits, ids, V);

@@ -12,6 +12,7 @@ int run_rope_store(const float *qkv, float *q_out, bf16_t *kc, bf16_t *vc, const
                    const float *sin_t, int B, int n_q, int n_kv, int D, int cap, int pos,
                    hipStream_t s);
 int run_argmax(const float *logits, int *ids, int B, int V, hipStream_t s);
+int run_argmax_tiles(const float *val, const int *idx, int *ids, int B, int n_tiles, hipStream_t s);
 int run_f32_to_bf16(const float *src, bf16_t *dst, size_t n, hipStream_t s);
 int run_fill_int(int *dst, int n, int value, hipStream_t s);
 int run_synth_bf16(bf16_t *dst, size_t n, uint64_t seed, float mean, float std, hipStream_t s);

@@ -148,6 +148,8 @@ int run_gemm(const GemmParams &p, bool gather, int epi, int rows_per_tile, int m
              hipStream_t s) {
   if (gather && epi == EPI_SWIGLU) return dispatch_rows<true, EPI_SWIGLU>(p, rows_per_tile, max_tiles, s);
   if (!gather && epi == EPI_F32) return dispatch_rows<false, EPI_F32>(p, rows_per_tile, max_tiles, s);
+  if (!gather && epi == EPI_ARGMAX && p.tiles == nullptr && p.amax_val && p.amax_idx)
+    return dispatch_rows<false, EPI_ARGMAX>(p, rows_per_tile, max_tiles, s);
   return fail(GPTOSS_ERR_DIM, "run_gemm: unsupported combination (gather=%d epi=%d)", (int)gather, epi);
 }
 

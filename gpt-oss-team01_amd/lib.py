@@ -19,6 +19,7 @@ PACK_SRC_FP32 = 1
 PACK_GLU = 2
 ENGINE_SYNTHETIC = 1
 ENGINE_PRECISE = 2
+ENGINE_LOGITS = 4
 
 
 class GptossError(RuntimeError):

@@ -226,13 +226,14 @@ class Engine:
     """Single-GPU decode engine over a flat ``.bin`` payload (or synthetic on-device weights)."""
 
     def __init__(self, cfg, weights_flat=None, max_batch=8, max_seq=64, synthetic=False,
-                 precise=False, seed=0):
+                 precise=False, seed=0, keep_logits=True):
         _need_gpu()
         import numpy as np
         self.L = _l.load()
         self.cfg = cfg
         self.max_batch, self.max_seq = max_batch, max_seq
-        flags = (_l.ENGINE_SYNTHETIC if synthetic else 0) | (_l.ENGINE_PRECISE if precise else 0)
+        flags = (_l.ENGINE_SYNTHETIC if synthetic else 0) | (_l.ENGINE_PRECISE if precise else 0) | \
+            (_l.ENGINE_LOGITS if keep_logits else 0)
         self._cc = _l.Config.from_config(cfg)
         wp = None
         if not synthetic:
@@ -269,6 +270,8 @@ class Engine:
         """fp32 [B, vocab] logits of the last step (copied to the host)."""
         lp, xp, nb = C.c_void_p(), C.c_void_p(), C.c_size_t()
         _l.check(self.L.gptoss_engine_debug_views(self._h, C.byref(lp), C.byref(xp), C.byref(nb)))
+        if not lp.value:
+            raise RuntimeError("the engine was created without keep_logits")
         V = self.cfg.vocab_size
         host = torch.empty(B, V, dtype=torch.float32)
         torch.cuda.synchronize()

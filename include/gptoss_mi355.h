@@ -200,6 +200,10 @@ typedef struct gptoss_engine gptoss_engine;
 
 enum {
   GPTOSS_ENGINE_SYNTHETIC = 1, /* host_weights ignored: N(0,0.02) bf16 weights generated on device */
+  GPTOSS_ENGINE_LOGITS = 4,    /* write the fp32 logits [B, vocab] of every step to memory (for
+                                  gptoss_engine_debug_views); without it the classifier GEMM keeps only
+                                  each row's arg-max, as max_logits_batched consumes them
+                                  (getp-csrc/src/model.cpp:144-148) */
   GPTOSS_ENGINE_PRECISE = 2    /* the reference CPU model's arithmetic (run.cpp:501-717) instead of the
                                   reference GPU path's bf16 staging: fp32 weights, activations and KV
                                   cache, double-accumulated dot products.  Reproduces the CPU model's

@@ -171,3 +171,23 @@ def test_engine_rejects_bad_arguments(ops, tiny):
     with pytest.raises(lib.GptossError):
         eng.step(np.zeros(2, np.int32), 16)           # position beyond max_seq
     eng.close()
+
+
+def test_fused_argmax_equals_argmax_of_logits(ops, tiny):
+    """Without GPTOSS_ENGINE_LOGITS the classifier GEMM keeps only each row's arg-max (two stages:
+    per column tile in the GEMM epilogue, then across tiles); the ids must equal those of the
+    engine that writes the logits and arg-maxes them, step for step, ties included."""
+    fx, cfg, flat = tiny
+    prompts = np.asarray(fx["prompts"], np.int32)
+    a = ops.Engine(cfg, flat, max_batch=8, max_seq=48, keep_logits=True)
+    b = ops.Engine(cfg, flat, max_batch=8, max_seq=48, keep_logits=False)
+    tok = prompts[:, 0].copy()
+    for pos in range(40):
+        na, nb = a.step(tok, pos), b.step(tok, pos)
+        assert np.array_equal(na, nb), pos
+        assert np.array_equal(na, a.last_logits(8).argmax(axis=1))
+        tok = na
+    with pytest.raises(RuntimeError):
+        b.last_logits(8)
+    a.close()
+    b.close()
