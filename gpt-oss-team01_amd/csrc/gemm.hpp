@@ -17,6 +17,8 @@ struct GemmParams {
   float *amax_val;     // EPI_ARGMAX (dense only): per (row, column tile) the largest value ...
   int *amax_idx;       // ... and the lowest column that holds it, [rows, n_col_tiles]
   const int *tiles;    // {n_tiles, (mat,row0,rows)*} or nullptr for a dense problem
+  const int *xcd_bounds;  // 9 positions in the tile list (tile << 16 | 16-bit fraction) that cut the
+                          // work into 8 parts of equal estimated cost, or nullptr: equal item counts
   int dense_rows;      // rows of the dense problem when tiles == nullptr
   int N, K;
   int n_col_tiles;     // gemm_col_tiles(N)
@@ -29,13 +31,16 @@ int run_gemm(const GemmParams &p, bool gather, int epi, int rows_per_tile, int m
              hipStream_t s);
 int run_combine(const float *y2, const float *topk_w, const int *inv_perm, float *out, int B, int H,
                 int k, int accumulate, hipStream_t s);
-int moe_rows_per_tile(int B, int k, int E);
+int moe_rows_per_tile(int B, int k, int E, bool mxfp4);
 int gemm_col_tiles(int N);  // column tiles of one workgroup's width
 // moe_route.hip
 int run_router(const void *t, const void *w_router, const float *b_router, float *logits, int B,
                int H, int E, int k, float *topk_w, int *topk_i, hipStream_t s);
 int run_topk_softmax(const float *logits, int B, int E, int k, float *topk_w, int *topk_i, hipStream_t s);
+// xcd_bounds (optional, 9 ints): see GemmParams; tile_cost0_x2 = twice the fixed part of a tile's
+// cost in units of one 32-row block of arithmetic (cost = fixed + number of 32-row blocks)
 int run_group(int B, int E, int k, float *topk_w, int *topk_i, int *expert_offsets,
-              int *sorted_pair_ids, int *inv_perm, int *tiles, int rows_per_tile, hipStream_t s);
+              int *sorted_pair_ids, int *inv_perm, int *tiles, int rows_per_tile, int *xcd_bounds,
+              int tile_cost0_x2, hipStream_t s);
 
 }  // namespace gptoss

@@ -133,6 +133,98 @@ __device__ __forceinline__ void w_load(WRing<NRING, FP4> &ring, const WStream &s
   }
 }
 
+// Epilogue of one wave's 32-column block at column n0: MB accumulator blocks of 32 rows starting
+// at row0, of which `rows` are real (rows <= 0: nothing is stored).
+// The MFMAs take the W fragment as their first operand, i.e. they compute the transposed tile:
+// a lane holds one token row (lane%32 of each 32-row block) and 16 of the wave's 32 output
+// channels, channel g*8 + h*4 + q in result register g*4 + q (h = lane/32).  Four consecutive
+// channels of a row are therefore four consecutive registers of one lane, which makes every
+// store 8 or 16 bytes wide and keeps each (gate, up) pair inside a lane.
+// Biases are wave-uniform per register and half-wave: they come in through scalar loads, which
+// do not queue behind the vector loads already in flight for the next item.
+template <int MB, int EPI>
+__device__ __forceinline__ void epilogue_store(const GemmParams &p, int mat, int row0, int rows, int n0,
+                                               int lane, const f32x16 (&acc)[MB]) {
+  const int N = p.N;
+  const int tok = lane & 31;
+  const bool hi = lane >= 32;
+  const int h4 = hi ? 4 : 0;
+  const float *bp = p.bias ? p.bias + (size_t)mat * N + n0 : nullptr;
+  if (EPI == EPI_SWIGLU) {
+    // channels 0-15 of the wave are the gates of pairs j0..j0+15, channels 16-31 their ups; in the
+    // unpacked matrix pair j is rows 2j (gate) and 2j+1 (up), so its biases are bp[2jj], bp[2jj+1]
+    const int half_n = N >> 1;
+    float bg[8], bu[8];
+#pragma unroll
+    for (int g = 0; g < 2; g++)
+#pragma unroll
+      for (int q = 0; q < 4; q++) {
+        const int jlo = g * 8 + q, jhi = jlo + 4;
+        const float g_lo = bp ? bp[2 * jlo] : 0.f, g_hi = bp ? bp[2 * jhi] : 0.f;
+        const float u_lo = bp ? bp[2 * jlo + 1] : 0.f, u_hi = bp ? bp[2 * jhi + 1] : 0.f;
+        bg[g * 4 + q] = hi ? g_hi : g_lo;
+        bu[g * 4 + q] = hi ? u_hi : u_lo;
+      }
+    // address = wave-uniform base (scalar registers) + a 32-bit per-lane element offset
+    bf16_t *o = reinterpret_cast<bf16_t *>(p.out) + (size_t)row0 * half_n + (n0 >> 1);
+    const uint32_t lane_off = (uint32_t)tok * (uint32_t)half_n + (uint32_t)h4;
+    const float L = p.limit;
+    const int row_lim = rows - tok;  // block i of this lane is a real row iff i*32 < row_lim
+#pragma unroll
+    for (int i = 0; i < MB; i++) {
+      if (i * 32 < row_lim) {
+        bf16_t *orow = o + (size_t)((uint32_t)(i * 32) * (uint32_t)half_n);
+#pragma unroll
+        for (int g = 0; g < 2; g++) {
+          float v[4];
+#pragma unroll
+          for (int q = 0; q < 4; q++) {
+            float gate = acc[i][g * 4 + q] + bg[g * 4 + q];
+            float up = acc[i][(g + 2) * 4 + q] + bu[g * 4 + q];
+            gate = fminf(gate, L);
+            up = fminf(fmaxf(up, -L), L);
+            // gate * sigmoid(1.702 gate) * (up + 1); exp2 and the hardware reciprocal are accurate
+            // to a few ulp of fp32, far inside the bf16 rounding of the result
+            const float e = __builtin_amdgcn_exp2f(-1.702f * 1.4426950408889634f * gate);
+            v[q] = gate * __builtin_amdgcn_rcpf(1.0f + e) * (up + 1.0f);
+          }
+          *reinterpret_cast<u32x2 *>(orow + lane_off + g * 8) =
+              u32x2{pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+        }
+      }
+    }
+  } else {
+    float bv[16];
+#pragma unroll
+    for (int g = 0; g < 4; g++)
+#pragma unroll
+      for (int q = 0; q < 4; q++) {
+        const float lo = bp ? bp[g * 8 + q] : 0.f, hi_v = bp ? bp[g * 8 + 4 + q] : 0.f;
+        bv[g * 4 + q] = hi ? hi_v : lo;
+      }
+    const uint32_t lane_off = (uint32_t)tok * (uint32_t)N + (uint32_t)h4;
+    const int row_lim = rows - tok;
+#pragma unroll
+    for (int i = 0; i < MB; i++) {
+      if (i * 32 < row_lim) {
+        const size_t row_off = (size_t)((uint32_t)(row0 + i * 32) * (uint32_t)N) + n0;
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+          float v[4];
+#pragma unroll
+          for (int q = 0; q < 4; q++) v[q] = acc[i][g * 4 + q] + bv[g * 4 + q];
+          if (EPI == EPI_F32)
+            *reinterpret_cast<f32x4 *>(reinterpret_cast<float *>(p.out) + row_off + lane_off + g * 8) =
+                f32x4{v[0], v[1], v[2], v[3]};
+          else
+            *reinterpret_cast<u32x2 *>(reinterpret_cast<bf16_t *>(p.out) + row_off + lane_off + g * 8) =
+                u32x2{pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+        }
+      }
+    }
+  }
+}
+
 // One (row tile, column tile) work item with a compile-time number of 32-row blocks, so every
 // loop below is fully unrolled and every global load of W is unconditional.  On entry the ring
 // holds slabs 0..NRING-2 of this item's W stream; while the last slabs are multiplied the ring is
@@ -318,100 +410,18 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, bf16_t *lds, int 
   }
   if (!wave_active) return;
 
-  // ---- epilogue ------------------------------------------------------------------------------
-  // The MFMAs take the W fragment as their first operand, i.e. they compute the transposed tile:
-  // a lane holds one token row (lane%32 of each 32-row block) and 16 of the wave's 32 output
-  // channels, channel g*8 + h*4 + q in result register g*4 + q (h = lane/32).  Four consecutive
-  // channels of a row are therefore four consecutive registers of one lane, which makes every
-  // store 8 or 16 bytes wide and keeps each (gate, up) pair inside a lane.
-  // Biases are wave-uniform per register and half-wave: they come in through scalar loads, which
-  // do not queue behind the vector loads already in flight for the next item.
-  const int tok = lane & 31;
-  const bool hi = lane >= 32;
-  const int h4 = hi ? 4 : 0;
-  const float *bp = p.bias ? p.bias + (size_t)mat * N + n0 : nullptr;
-  if (EPI == EPI_SWIGLU) {
-    // channels 0-15 of the wave are the gates of pairs j0..j0+15, channels 16-31 their ups; in the
-    // unpacked matrix pair j is rows 2j (gate) and 2j+1 (up), so its biases are bp[2jj], bp[2jj+1]
-    const int half_n = N >> 1;
-    float bg[8], bu[8];
-#pragma unroll
-    for (int g = 0; g < 2; g++)
-#pragma unroll
-      for (int q = 0; q < 4; q++) {
-        const int jlo = g * 8 + q, jhi = jlo + 4;
-        const float g_lo = bp ? bp[2 * jlo] : 0.f, g_hi = bp ? bp[2 * jhi] : 0.f;
-        const float u_lo = bp ? bp[2 * jlo + 1] : 0.f, u_hi = bp ? bp[2 * jhi + 1] : 0.f;
-        bg[g * 4 + q] = hi ? g_hi : g_lo;
-        bu[g * 4 + q] = hi ? u_hi : u_lo;
-      }
-    // address = wave-uniform base (scalar registers) + a 32-bit per-lane element offset
-    bf16_t *o = reinterpret_cast<bf16_t *>(p.out) + (size_t)row0 * half_n + (n0 >> 1);
-    const uint32_t lane_off = (uint32_t)tok * (uint32_t)half_n + (uint32_t)h4;
-    const float L = p.limit;
-    const int row_lim = rows - tok;  // block i of this lane is a real row iff i*32 < row_lim
-#pragma unroll
-    for (int i = 0; i < MB; i++) {
-      if (i * 32 < row_lim) {
-        bf16_t *orow = o + (size_t)((uint32_t)(i * 32) * (uint32_t)half_n);
-#pragma unroll
-        for (int g = 0; g < 2; g++) {
-          float v[4];
-#pragma unroll
-          for (int q = 0; q < 4; q++) {
-            float gate = acc[i][g * 4 + q] + bg[g * 4 + q];
-            float up = acc[i][(g + 2) * 4 + q] + bu[g * 4 + q];
-            gate = fminf(gate, L);
-            up = fminf(fmaxf(up, -L), L);
-            // gate * sigmoid(1.702 gate) * (up + 1); exp2 and the hardware reciprocal are accurate
-            // to a few ulp of fp32, far inside the bf16 rounding of the result
-            const float e = __builtin_amdgcn_exp2f(-1.702f * 1.4426950408889634f * gate);
-            v[q] = gate * __builtin_amdgcn_rcpf(1.0f + e) * (up + 1.0f);
-          }
-          *reinterpret_cast<u32x2 *>(orow + lane_off + g * 8) =
-              u32x2{pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
-        }
-      }
-    }
-  } else {
-    float bv[16];
-#pragma unroll
-    for (int g = 0; g < 4; g++)
-#pragma unroll
-      for (int q = 0; q < 4; q++) {
-        const float lo = bp ? bp[g * 8 + q] : 0.f, hi_v = bp ? bp[g * 8 + 4 + q] : 0.f;
-        bv[g * 4 + q] = hi ? hi_v : lo;
-      }
-    const uint32_t lane_off = (uint32_t)tok * (uint32_t)N + (uint32_t)h4;
-    const int row_lim = rows - tok;
-#pragma unroll
-    for (int i = 0; i < MB; i++) {
-      if (i * 32 < row_lim) {
-        const size_t row_off = (size_t)((uint32_t)(row0 + i * 32) * (uint32_t)N) + n0;
-#pragma unroll
-        for (int g = 0; g < 4; g++) {
-          float v[4];
-#pragma unroll
-          for (int q = 0; q < 4; q++) v[q] = acc[i][g * 4 + q] + bv[g * 4 + q];
-          if (EPI == EPI_F32)
-            *reinterpret_cast<f32x4 *>(reinterpret_cast<float *>(p.out) + row_off + lane_off + g * 8) =
-                f32x4{v[0], v[1], v[2], v[3]};
-          else
-            *reinterpret_cast<u32x2 *>(reinterpret_cast<bf16_t *>(p.out) + row_off + lane_off + g * 8) =
-                u32x2{pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
-        }
-      }
-    }
-  }
+  epilogue_store<MB, EPI>(p, mat, row0, rows, n0, lane, acc);
 }
 
 // NRING: slabs of W held in registers per wave, NRING-1 of them in flight.
 constexpr int GEMM_NRING = 3;
 
 // Persistent kernel: the grid is one workgroup of 8 waves per CU; workgroups are dealt round-robin
-// to the 8 XCDs, XCD x owns the x-th contiguous eighth of the work list (consecutive column tiles
+// to the 8 XCDs, XCD x owns the x-th contiguous part of the work list (consecutive column tiles
 // of the same expert, so that expert's rows stay in that XCD's L2) and its workgroups walk that
-// eighth with a stride of the number of workgroups per XCD.
+// part with a stride of the number of workgroups per XCD.  The parts hold equal numbers of items,
+// or, when the grouping kernel supplied cut positions, equal estimated cost (experts with many
+// rows next to experts with few would otherwise leave some XCDs idle early).
 template <int MBMAX, bool GATHER, int EPI, bool FP4>
 __global__ __launch_bounds__(GEMM_THREADS, 2) void grouped_gemm_kernel(GemmParams p) {
   constexpr int BM = MBMAX * 32;
@@ -423,18 +433,27 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void grouped_gemm_kernel(GemmParam
 
   const int n_tiles = p.tiles ? p.tiles[0] : (p.dense_rows + BM - 1) / BM;
   const int total = n_tiles * p.n_col_tiles;
-  const int chunk = (total + 7) >> 3;
   const int per_xcd = gridDim.x >> 3;
   const int xcd = blockIdx.x & 7;
+  int lo, hi;  // this XCD's part of the work list
+  if (p.xcd_bounds) {
+    auto item = [&](int b) { return (b >> 16) * p.n_col_tiles + (((b & 0xffff) * p.n_col_tiles) >> 16); };
+    lo = item(p.xcd_bounds[xcd]);
+    hi = item(p.xcd_bounds[xcd + 1]);
+  } else {
+    const int chunk = (total + 7) >> 3;
+    lo = xcd * chunk;
+    hi = min(total, lo + chunk);
+  }
   int j = blockIdx.x >> 3;
-  auto valid = [&](int jj) { return jj < chunk && xcd * chunk + jj < total; };
+  auto valid = [&](int jj) { return lo + jj < hi; };
   if (!valid(j)) return;
 
   struct Item {
     int mat, row0, rows, ct;
   };
   auto decode = [&](int jj) {
-    const int work = xcd * chunk + jj;
+    const int work = lo + jj;
     const int tile = work / p.n_col_tiles;
     Item it;
     it.ct = work - tile * p.n_col_tiles;

@@ -10,7 +10,7 @@ namespace gptoss {
 
 struct MoeWorkspace {
   float *logits, *topk_w;
-  int *topk_i, *expert_offsets, *sorted_pair_ids, *inv_perm, *tiles;
+  int *topk_i, *expert_offsets, *sorted_pair_ids, *inv_perm, *tiles, *xcd_bounds;
   bf16_t *act;
   float *y2;
   size_t bytes;
@@ -32,6 +32,7 @@ static MoeWorkspace carve(void *base, int B, int E, int k, int H, int I) {
   w.sorted_pair_ids = (int *)take(P * 4);
   w.inv_perm = (int *)take(P * 4);
   w.tiles = (int *)take((1 + 3 * (P / 32 + E)) * 4);
+  w.xcd_bounds = (int *)take(16 * 4);
   w.act = (bf16_t *)take(P * I * 2);
   w.y2 = (float *)take(P * H * 4);
   w.bytes = off;
@@ -41,14 +42,23 @@ static MoeWorkspace carve(void *base, int B, int E, int k, int H, int I) {
 // Row-tile size (32, 64, 128 or 160 rows) for B*k pairs over E experts: the smallest tile that holds an average
 // expert's rows plus 2.5 standard deviations of a uniform routing, so that nearly every expert is
 // a single tile (its weights are then streamed exactly once).
-int moe_rows_per_tile(int B, int k, int E) {
+int moe_rows_per_tile(int B, int k, int E, bool mxfp4) {
   double avg = (double)B * k / E;
   double need = avg + 2.5 * sqrt(avg);
+
   if (need <= 32) return 32;
   if (need <= 64) return 64;
   if (need <= 128) return 128;
   return 160;
 }
+
+// Fixed part of a work item's cost, in half units of one 32-row block of arithmetic, used to cut
+// the work list into 8 equally expensive parts.  With bf16 weights an item is dominated by
+// streaming its 1.5 MB of W whatever its row count (16 + blocks); with MXFP4 weights, a quarter of
+// the bytes, the arithmetic weighs more (5 + blocks).  Both constants are the measured optimum on a
+// Zipf-skewed routing; a uniform routing is indifferent to them.
+constexpr int MOE_TILE_COST0_X2_BF16 = 32;
+constexpr int MOE_TILE_COST0_X2_MXFP4 = 10;
 
 static int check_moe(const gptoss_moe_weights *w, const void *t, int B, float *out, void *ws,
                      size_t ws_bytes) {
@@ -108,14 +118,15 @@ static int moe_forward_impl(const gptoss_moe_weights *w, const void *t, int B, f
   const int E = w->n_experts, k = w->top_k, H = w->hidden, I = w->intermediate;
   hipStream_t s = (hipStream_t)stream;
   MoeWorkspace ws = carve(workspace, B, E, k, H, I);
-  const int rpt = moe_rows_per_tile(B, k, E);
+  const int rpt = moe_rows_per_tile(B, k, E, mxfp4 != 0);
   const int max_tiles = gptoss_moe_max_tiles(B, k, E, rpt);
 
   // router GEMM with the gating of its own 16 tokens fused in, then the stable grouping
   rc = run_router(t, w->w_router, w->b_router, ws.logits, B, H, E, k, ws.topk_w, ws.topk_i, s);
   if (rc != GPTOSS_OK) return rc;
   rc = run_group(B, E, k, ws.topk_w, ws.topk_i, ws.expert_offsets, ws.sorted_pair_ids, ws.inv_perm,
-                 ws.tiles, rpt, s);
+                 ws.tiles, rpt, ws.xcd_bounds, mxfp4 ? MOE_TILE_COST0_X2_MXFP4 : MOE_TILE_COST0_X2_BF16, s);
+  const int *bounds = max_tiles < 32768 ? ws.xcd_bounds : nullptr;
   if (rc != GPTOSS_OK) return rc;
 
   GemmParams g1{};
@@ -127,6 +138,7 @@ static int moe_forward_impl(const gptoss_moe_weights *w, const void *t, int B, f
   g1.bias = w->b1;
   g1.out = ws.act;
   g1.tiles = ws.tiles;
+  g1.xcd_bounds = bounds;
   g1.N = 2 * I;
   g1.K = H;
   g1.n_col_tiles = gemm_col_tiles(2 * I);
@@ -141,6 +153,7 @@ static int moe_forward_impl(const gptoss_moe_weights *w, const void *t, int B, f
   g2.bias = w->b2;
   g2.out = ws.y2;
   g2.tiles = ws.tiles;
+  g2.xcd_bounds = bounds;
   g2.N = H;
   g2.K = I;
   g2.n_col_tiles = gemm_col_tiles(H);

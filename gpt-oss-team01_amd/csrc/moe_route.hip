@@ -211,7 +211,7 @@ __device__ __forceinline__ int wave_scan4(const int (&v)[4], int (&ex)[4]) {
 __global__ __launch_bounds__(SORT_THREADS) void group_sort_kernel(
     const int *__restrict__ topk_i, int P, int E, int nbits, int *__restrict__ expert_offsets,
     int *__restrict__ sorted_pair_ids, int *__restrict__ inv_perm, int *__restrict__ tiles,
-    int rows_per_tile) {
+    int rows_per_tile, int *__restrict__ xcd_bounds, int cost0) {
   extern __shared__ int smem[];
   int *hist = smem;                    // [SORT_WAVES][E] per-wave counts, then per-wave cursors
   int *total = hist + SORT_WAVES * E;  // [E]
@@ -296,6 +296,38 @@ __global__ __launch_bounds__(SORT_THREADS) void group_sort_kernel(
       expert_offsets[E] = all;
       if (tiles != nullptr && rows_per_tile > 0) tiles[0] = n_tiles;
     }
+    // Where to cut the tile list into 8 parts (one per XCD) of equal estimated cost: a tile costs
+    // cost0 + 2 per 32-row block (half units), all work items of a tile cost the same, and a cut may
+    // fall inside a tile (between two of its column tiles), hence the 16-bit fraction.
+    if (xcd_bounds != nullptr && tiles != nullptr && rows_per_tile > 0) {
+      const int cfull = cost0 + 2 * (rows_per_tile / 32);
+      int cost[4], clast[4], cpre[4];
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const int last_rows = cnt[i] - (nt[i] - 1) * rows_per_tile;
+        clast[i] = cost0 + 2 * ((last_rows + 31) / 32);
+        cost[i] = (nt[i] > 0) ? (nt[i] - 1) * cfull + clast[i] : 0;
+      }
+      const int ctot = wave_scan4(cost, cpre);
+      for (int x = 0; x < 8; x++) {
+        const int target = (int)((long long)x * ctot / 8);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          if (cost[i] > 0 && cpre[i] <= target && target < cpre[i] + cost[i]) {
+            const int t = min((target - cpre[i]) / cfull, nt[i] - 1);
+            const int rest = target - cpre[i] - t * cfull;
+            const int ct = (t == nt[i] - 1) ? clast[i] : cfull;
+            const int frac = min(65535, (int)(((long long)rest << 16) / ct));
+            xcd_bounds[x] = ((tile_ex[i] + t) << 16) | frac;
+          }
+        }
+      }
+      if (lane == 0) {
+        xcd_bounds[8] = n_tiles << 16;
+        if (ctot == 0)
+          for (int x = 0; x < 8; x++) xcd_bounds[x] = 0;
+      }
+    }
   }
   __syncthreads();
 
@@ -374,26 +406,28 @@ extern "C" int gptoss_moe_max_tiles(int B, int k, int E, int rows_per_tile) {
 
 static int moe_route_impl(const float *logits, int B, int E, int k, float *topk_w, int *topk_i,
                           int *expert_offsets, int *sorted_pair_ids, int *inv_perm, int *tiles,
-                          int rows_per_tile, void *stream, bool gate);
+                          int rows_per_tile, int *xcd_bounds, int tile_cost0_x2, void *stream, bool gate);
 
 // grouping only: topk_i was already written by the fused router kernel
 int gptoss::run_group(int B, int E, int k, float *topk_w, int *topk_i, int *expert_offsets,
                       int *sorted_pair_ids, int *inv_perm, int *tiles, int rows_per_tile,
-                      hipStream_t s) {
+                      int *xcd_bounds, int tile_cost0_x2, hipStream_t s) {
+  // the cut positions hold the tile index in 15 bits
+  if (gptoss_moe_max_tiles(B, k, E, rows_per_tile) >= 32768) xcd_bounds = nullptr;
   return moe_route_impl(nullptr, B, E, k, topk_w, topk_i, expert_offsets, sorted_pair_ids, inv_perm,
-                        tiles, rows_per_tile, s, false);
+                        tiles, rows_per_tile, xcd_bounds, tile_cost0_x2, s, false);
 }
 
 extern "C" int gptoss_moe_route(const float *logits, int B, int E, int k, float *topk_w,
                                 int *topk_i, int *expert_offsets, int *sorted_pair_ids,
                                 int *inv_perm, int *tiles, int rows_per_tile, void *stream) {
   return moe_route_impl(logits, B, E, k, topk_w, topk_i, expert_offsets, sorted_pair_ids, inv_perm,
-                        tiles, rows_per_tile, stream, true);
+                        tiles, rows_per_tile, nullptr, 0, stream, true);
 }
 
 static int moe_route_impl(const float *logits, int B, int E, int k, float *topk_w, int *topk_i,
                           int *expert_offsets, int *sorted_pair_ids, int *inv_perm, int *tiles,
-                          int rows_per_tile, void *stream, bool gate) {
+                          int rows_per_tile, int *xcd_bounds, int tile_cost0_x2, void *stream, bool gate) {
   GPTOSS_REQUIRE(expert_offsets, GPTOSS_ERR_NULL, "moe_route: null pointer");
   GPTOSS_REQUIRE(B <= 0 || ((logits || !gate) && topk_w && topk_i && sorted_pair_ids && inv_perm),
                  GPTOSS_ERR_NULL, "moe_route: null pointer");
@@ -415,7 +449,8 @@ static int moe_route_impl(const float *logits, int B, int E, int k, float *topk_
     TraceScope ts("group_sort", s);
     group_sort_kernel<<<1, SORT_THREADS, smem, s>>>(topk_i, B * k, E, nbits, expert_offsets,
                                                     sorted_pair_ids, inv_perm,
-                                                    rows_per_tile ? tiles : nullptr, rows_per_tile);
+                                                    rows_per_tile ? tiles : nullptr, rows_per_tile,
+                                                    xcd_bounds, tile_cost0_x2);
   }
   GPTOSS_LAUNCH_CHECK("group_sort_kernel");
   return GPTOSS_OK;

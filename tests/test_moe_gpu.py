@@ -164,3 +164,35 @@ def test_moe_forward_accumulate_and_determinism(ops):
     y = x.clone()
     layer.forward(t, out=y, accumulate=True)
     assert torch.equal(y, x + a)
+
+
+@pytest.mark.parametrize("B,E,H,I", [(3000, 16, 256, 512), (1500, 64, 512, 256)])
+def test_moe_forward_skewed_routing_is_batch_invariant(ops, orc, B, E, H, I):
+    """Zipf-skewed routing (experts with many row tiles next to experts with a few rows): the work
+    list is then cut into per-XCD parts by estimated cost, with cuts that fall inside tiles.  Every
+    token's output must not depend on what else is in the batch: the full batch equals, bit for bit,
+    the same tokens run in two halves (other tiles, other cuts), and a sample equals the oracle."""
+    L = _rand_layer(E, H, I, 21)
+    ranks = np.random.default_rng(B).permutation(E) + 1
+    L["b_router"] = torch.from_numpy((1.5 * np.log(1.0 / ranks ** 1.1)).astype(np.float32))
+    g = torch.Generator().manual_seed(B)
+    t = _bf16(torch.randn(B, H, generator=g))
+    layer = ops.MoeLayer(*[L[n].cuda() for n in ("w_router", "b_router", "w1", "b1", "w2", "b2")],
+                         max_tokens=B)
+    full = layer.forward(t.cuda()).clone()
+    logits, tw, ti, off, srt, inv = [x.cpu().numpy() for x in layer.routing_views()]
+    counts = np.diff(off)
+    assert counts.max() >= 4 * counts.mean() and counts.max() > 3 * 160   # several tiles for one expert
+    h = B // 2 + 7
+    first = layer.forward(t[:h].cuda()).clone()
+    second = layer.forward(t[h:].cuda()).clone()
+    assert torch.equal(full[:h], first)
+    assert torch.equal(full[h:], second)
+    n_chk = 40
+    want, _, _, oti = orc.moe_layer(_f32np(t)[:n_chk], *[_f32np(L[n]) for n in
+                                    ("w_router", "b_router", "w1", "b1", "w2", "b2")],
+                                    k=4, limit=7.0, stage=orc.STAGE_SWIGLU, want_routing=True)
+    same = (oti == ti[:n_chk]).all(axis=1)
+    assert same.mean() > 0.9
+    mx, mean = rel_errors(full.cpu().numpy()[:n_chk][same], want[same])
+    assert mx <= TOL_MAX and mean <= TOL_MEAN, (mx, mean)
