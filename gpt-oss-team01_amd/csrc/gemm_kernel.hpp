@@ -39,41 +39,21 @@ constexpr int BK = 64;            // k per LDS slab (4 MFMA k-steps)
 constexpr int LDS_ROW = BK + 8;   // padded row length in bf16 elements (144 B)
 constexpr int BN = GEMM_WAVES * 32;  // columns per workgroup
 
-// MXFP4 operand expansion.  One dword holds the lane's 8 e2m1 codes of a k-step (element j < 4 in
-// the low nibble of byte j, element j >= 4 in the high nibble of byte j-4).  tab[] holds the eight
-// positive bf16 magnitudes already multiplied by the block's power-of-two scale, as byte tables
-// for v_perm_b32: tab[0]/tab[1] = low bytes of entries 0-3 / 4-7, tab[2]/tab[3] = high bytes.
-struct Fp4Table {
-  uint32_t lo_a, lo_b, hi_a, hi_b;
-};
+// MXFP4 operand expansion.  One dword holds the lane's 8 e2m1 codes of a k-step in checkpoint
+// order (byte j = elements 2j in the low and 2j+1 in the high nibble), which is what the hardware
+// conversion takes: v_cvt_scalef32_pk_bf16_fp4 turns one byte into the bf16 pair (value * scale),
+// exact for a power-of-two scale inside the bf16 normal range.
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 
-__device__ __forceinline__ Fp4Table fp4_table(uint32_t e8m0) {
-  // bf16 bit patterns of 0, .5 | 1, 1.5 | 2, 3 | 4, 6 as pairs; the exponent field starts at bit 7
-  // d * 0x00800080 adds d to both exponent fields: for negative d the borrow out of the low half
-  // is undone by the carry of the low-half addition below
-  const uint32_t dd = (e8m0 - 127u) * 0x00800080u;
-  const uint32_t t01 = 0x3F000000u + ((e8m0 - 127u) << 23);  // entry 0 stays +0
-  const uint32_t t23 = 0x3FC03F80u + dd;
-  const uint32_t t45 = 0x40404000u + dd;
-  const uint32_t t67 = 0x40C04080u + dd;
-  Fp4Table t;
-  // v_perm_b32(S0, S1, sel): selector values 0-3 pick bytes of S1, 4-7 bytes of S0
-  t.lo_a = __builtin_amdgcn_perm(t23, t01, 0x06040200u);
-  t.hi_a = __builtin_amdgcn_perm(t23, t01, 0x07050301u);
-  t.lo_b = __builtin_amdgcn_perm(t67, t45, 0x06040200u);
-  t.hi_b = __builtin_amdgcn_perm(t67, t45, 0x07050301u);
-  return t;
+__device__ __forceinline__ float fp4_scale(uint32_t e8m0) {
+  return __builtin_bit_cast(float, e8m0 << 23);  // 2^(e8m0 - 127)
 }
 
-__device__ __forceinline__ u32x4 fp4_expand(uint32_t w, const Fp4Table &t) {
-  const uint32_t m_lo = w & 0x07070707u, m_hi = (w >> 4) & 0x07070707u;
-  uint32_t l0 = __builtin_amdgcn_perm(t.lo_b, t.lo_a, m_lo);
-  uint32_t h0 = __builtin_amdgcn_perm(t.hi_b, t.hi_a, m_lo) | ((w << 4) & 0x80808080u);
-  uint32_t l1 = __builtin_amdgcn_perm(t.lo_b, t.lo_a, m_hi);
-  uint32_t h1 = __builtin_amdgcn_perm(t.hi_b, t.hi_a, m_hi) | (w & 0x80808080u);
-  // interleave low and high bytes into bf16 pairs: elements 0,1 | 2,3 | 4,5 | 6,7
-  return u32x4{__builtin_amdgcn_perm(h0, l0, 0x05010400u), __builtin_amdgcn_perm(h0, l0, 0x07030602u),
-               __builtin_amdgcn_perm(h1, l1, 0x05010400u), __builtin_amdgcn_perm(h1, l1, 0x07030602u)};
+__device__ __forceinline__ u32x4 fp4_expand(uint32_t w, float scale) {
+  return u32x4{__builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, scale, 0)),
+               __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, scale, 1)),
+               __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, scale, 2)),
+               __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, scale, 3))};
 }
 
 template <int I, int N, typename F>
@@ -287,10 +267,10 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, bf16_t *lds, int 
   auto compute = [&](int stage, auto rsel) {
     constexpr int R = decltype(rsel)::value;
     const bf16_t *base = a_src + stage * LDS_STAGE;
-    Fp4Table tab[2];
+    float scale[2] = {0.f, 0.f};  // of k 0-31 and k 32-63 of the slab
     if (FP4) {
-      tab[0] = fp4_table(ring.s[R] & 0xffu);
-      tab[1] = fp4_table((ring.s[R] >> 8) & 0xffu);
+      scale[0] = fp4_scale(ring.s[R] & 0xffu);
+      scale[1] = fp4_scale((ring.s[R] >> 8) & 0xffu);
     }
     // af[0] already holds the fragments of k-step 0 (requested before the previous barrier).  The
     // fragments of k-step kk+1 are requested before the MFMAs of k-step kk are issued, and the
@@ -304,7 +284,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, bf16_t *lds, int 
               as_bf16x8(*reinterpret_cast<const u32x4 *>(base + i * 32 * LDS_ROW + (kk + 1) * 16));
       }
       bf16x8 b;
-      if (FP4) b = as_bf16x8(fp4_expand(ring.b[R][0][kk], tab[kk >> 1]));
+      if (FP4) b = as_bf16x8(fp4_expand(ring.b[R][0][kk], scale[kk >> 1]));
       else b = as_bf16x8(ring.b[R][kk % BQ]);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll

@@ -108,14 +108,7 @@ __global__ __launch_bounds__(256) void pack_mxfp4_kernel(const unsigned char *__
 #pragma unroll
   for (int kk = 0; kk < 4; kk++) {
     const int k0 = (slab * 4 + kk) * 16 + (lane >> 5) * 8;  // the lane's 8 consecutive k
-    uint32_t src = *reinterpret_cast<const uint32_t *>(brow + k0 / 2);  // nibble j = element k0+j
-    uint32_t o = 0;
-#pragma unroll
-    for (int j = 0; j < 8; j++) {
-      uint32_t code = (src >> (4 * j)) & 0xfu;
-      o |= code << ((j < 4) ? (8 * j) : (8 * (j - 4) + 4));
-    }
-    w[kk] = o;
+    w[kk] = *reinterpret_cast<const uint32_t *>(brow + k0 / 2);  // nibble j = element k0+j
   }
   *reinterpret_cast<u32x4 *>(md + (item * 64 + lane) * 16) = u32x4{w[0], w[1], w[2], w[3]};
   if (lane < 32) {
