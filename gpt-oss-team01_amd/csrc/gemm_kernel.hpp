@@ -241,19 +241,25 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, bf16_t *lds, int 
     }
     a_off[i] = (uint32_t)src * (uint32_t)K + a_kc * 8;
   }
-  u32x4 areg[AC];
-  auto load_a = [&](int s) {
+  // Register sets for A in flight.  With bf16 weights a slab's rows are requested one iteration
+  // before they are stored to LDS; with MXFP4 weights the iterations are short (a quarter of the
+  // W bytes), so two sets alternate and every request has two iterations to complete.
+  constexpr int APF = FP4 ? 2 : 1;
+  u32x4 areg[APF][AC];
+  auto load_a = [&](int s, auto psel) {
+    constexpr int P = decltype(psel)::value % APF;
 #pragma unroll
     for (int i = 0; i < AC; i++)
-      if (a_live[i]) areg[i] = *reinterpret_cast<const u32x4 *>(p.A + a_off[i] + s * BK);
+      if (a_live[i]) areg[P][i] = *reinterpret_cast<const u32x4 *>(p.A + a_off[i] + s * BK);
   };
   bf16_t *a_dst = lds + a_row * LDS_ROW + a_kc * 8;
-  auto store_a = [&](int stage, bool zero) {
+  auto store_a = [&](int stage, bool zero, auto psel) {
+    constexpr int P = decltype(psel)::value % APF;
 #pragma unroll
     for (int i = 0; i < AC; i++)
       if (a_live[i])
         *reinterpret_cast<u32x4 *>(a_dst + stage * LDS_STAGE + APASS * i * LDS_ROW) =
-            zero ? u32x4{0u, 0u, 0u, 0u} : areg[i];
+            zero ? u32x4{0u, 0u, 0u, 0u} : areg[P][i];
   };
 
   f32x16 acc[MB];
@@ -307,16 +313,27 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, bf16_t *lds, int 
   // item; the (at most NRING-1) padding iterations multiply zero A rows.
   const int last = nslab - 1;
   const int padded = (nslab + NRING - 1) / NRING * NRING;
-  load_a(0);
-  store_a(0, false);
-  load_a(min(1, last));
-  store_a(1, nslab <= 1);
-  load_a(min(2, last));
+  using P0 = std::integral_constant<int, 0>;
+  using P1 = std::integral_constant<int, 1>;
+  if constexpr (APF == 2) {
+    load_a(0, P0{});
+    load_a(min(1, last), P1{});
+    store_a(0, false, P0{});
+    store_a(1, nslab <= 1, P1{});
+    load_a(min(2, last), P0{});
+    load_a(min(3, last), P1{});
+  } else {
+    load_a(0, P0{});
+    store_a(0, false, P0{});
+    load_a(min(1, last), P0{});
+    store_a(1, nslab <= 1, P0{});
+    load_a(min(2, last), P0{});
+  }
   __syncthreads();
   read_first_frags(0);
 
   int st = 0;  // s % 3
-  auto body = [&](int s, auto rsel) {
+  auto body = [&](int s, auto rsel, auto psel) {
     constexpr int R = decltype(rsel)::value;
     using Refill = std::integral_constant<int, (R + D) % NRING>;
     // ring slot consumed at iteration s+D: slab s+D of this item, nothing useful while padding,
@@ -326,14 +343,30 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, bf16_t *lds, int 
     w_load<NRING, FP4>(ring, wrap ? next : cur, min(wrap ? t - padded : t, last), lane, Refill{});
     compute(st, rsel);
     const int st1 = (st == 2) ? 0 : st + 1, st2 = (st1 == 2) ? 0 : st1 + 1;
-    store_a(st2, s + 2 >= nslab);  // rows of slab s+2 (zeros while padding)
-    load_a(min(s + 3, last));
+    store_a(st2, s + 2 >= nslab, psel);  // rows of slab s+2 (zeros while padding)
+    load_a(min(s + 2 + APF, last), psel);
     read_first_frags(st1);
     st = st1;
     __syncthreads();
   };
-  for (int s = 0; s < padded; s += NRING)
-    static_for<0, NRING>([&](auto r) { body(s + (int)decltype(r)::value, r); });
+  if constexpr (APF == 2) {
+    // the register set alternates with the parity of s: pairs of NRING-iteration groups, then one
+    // more group when their number is odd
+    int s = 0;
+    for (; s + 2 * NRING <= padded; s += 2 * NRING)
+      static_for<0, 2 * NRING>([&](auto r) {
+        constexpr int Q = decltype(r)::value;
+        body(s + Q, std::integral_constant<int, Q % NRING>{}, std::integral_constant<int, Q & 1>{});
+      });
+    if (s < padded)
+      static_for<0, NRING>([&](auto r) {
+        constexpr int Q = decltype(r)::value;
+        body(s + Q, std::integral_constant<int, Q>{}, std::integral_constant<int, Q & 1>{});
+      });
+  } else {
+    for (int s = 0; s < padded; s += NRING)
+      static_for<0, NRING>([&](auto r) { body(s + (int)decltype(r)::value, r, P0{}); });
+  }
 
   if (EPI == EPI_ARGMAX) {
     // Row-wise arg-max of this workgroup's 256 columns without writing the products: every lane

@@ -309,17 +309,29 @@ __global__ __launch_bounds__(SORT_THREADS) void group_sort_kernel(
         cost[i] = (nt[i] > 0) ? (nt[i] - 1) * cfull + clast[i] : 0;
       }
       const int ctot = wave_scan4(cost, cpre);
+      const float rcp_cfull = __builtin_amdgcn_rcpf((float)cfull);
+      // all quantities fit 32 bits: ctot < 2^15 tiles * (cost0 + 16)
       for (int x = 0; x < 8; x++) {
-        const int target = (int)((long long)x * ctot / 8);
+        const int target = (x * ctot) >> 3;
+        int pre = -1, nte = 0, cl = 0, te = 0;  // the (at most one) expert of this lane that holds the cut
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-          if (cost[i] > 0 && cpre[i] <= target && target < cpre[i] + cost[i]) {
-            const int t = min((target - cpre[i]) / cfull, nt[i] - 1);
-            const int rest = target - cpre[i] - t * cfull;
-            const int ct = (t == nt[i] - 1) ? clast[i] : cfull;
-            const int frac = min(65535, (int)(((long long)rest << 16) / ct));
-            xcd_bounds[x] = ((tile_ex[i] + t) << 16) | frac;
-          }
+          const bool hit = cost[i] > 0 && cpre[i] <= target && target < cpre[i] + cost[i];
+          pre = hit ? cpre[i] : pre;
+          nte = hit ? nt[i] : nte;
+          cl = hit ? clast[i] : cl;
+          te = hit ? tile_ex[i] : te;
+        }
+        if (pre >= 0) {
+          // float quotient (operands < 2^24) with a one-step correction instead of integer division
+          const int a = target - pre;
+          int t = (int)((float)a * rcp_cfull);
+          t -= (t * cfull > a) ? 1 : 0;
+          t += ((t + 1) * cfull <= a) ? 1 : 0;
+          t = min(t, nte - 1);
+          const int rest = a - t * cfull;
+          const float inv = (t == nte - 1) ? __builtin_amdgcn_rcpf((float)cl) : rcp_cfull;
+          xcd_bounds[x] = ((te + t) << 16) | min(65535, (int)((float)rest * 65536.0f * inv));
         }
       }
       if (lane == 0) {
