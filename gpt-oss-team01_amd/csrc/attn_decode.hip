@@ -14,6 +14,7 @@
 //     contiguous per load; position p lives in slot p % capacity (ring buffer for window layers);
 //   * long contexts are cut into chunks (flash-decoding): partial (max, sum, O) per chunk, merged
 //     with the sink by a small second kernel; sequences that fit one chunk finish in the first.
+#include <algorithm>
 #include <type_traits>
 
 #include "common.hpp"
@@ -32,17 +33,22 @@ struct AttnParams {
   bf16_t *out;         // [B, n_q, D]
   float *part_o;       // [B, max_chunks, n_q, D]
   float *part_ml;      // [B, max_chunks, n_q, 2]
-  int B, n_q, n_kv, G, cap, window, chunk, max_chunks, max_len;
+  int B, n_q, n_kv, G, cap, window, max_chunks, max_len;
+  int rows_per_seq;    // query rows per cached sequence: row b reads the cache of sequence b / rows_per_seq
   float scale_log2e;   // log2(e) / sqrt(D)
 };
 
 struct SeqRange {
   int s_begin, s_end;  // slot range to visit (s_begin is a multiple of 64)
   int t_lo, len;       // active positions are [t_lo, len)
-  int nchunks;
+  int chunk, nchunks;  // slots per work item, number of work items
 };
 
-__device__ __forceinline__ SeqRange seq_range(int len, int cap, int window, int chunk, int max_len) {
+// Slots per work item as a function of the row's own slot range, so that a row's result does not
+// depend on what else is in the launch (one lock-step position or many positions of a prefill).
+__host__ __device__ __forceinline__ int attn_chunk_tokens(int span) { return span > 1024 ? 512 : 256; }
+
+__device__ __forceinline__ SeqRange seq_range(int len, int cap, int window, int max_len) {
   SeqRange r;
   len = max(0, min(len, max_len));
   r.len = len;
@@ -55,7 +61,8 @@ __device__ __forceinline__ SeqRange seq_range(int len, int cap, int window, int 
     r.s_begin = 0;
     r.s_end = cap;
   }
-  r.nchunks = max(1, (r.s_end - r.s_begin + chunk - 1) / chunk);
+  r.chunk = attn_chunk_tokens(r.s_end - r.s_begin);
+  r.nchunks = max(1, (r.s_end - r.s_begin + r.chunk - 1) / r.chunk);
   return r;
 }
 
@@ -73,7 +80,7 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
   // the chip is still filling and the grid ends on chunk 0, which every sequence has
   const int chunk_id = p.max_chunks - 1 - rest / p.B;
   if (chunk_id < 0) return;
-  const SeqRange r = seq_range(__builtin_amdgcn_readfirstlane(p.lens[b]), p.cap, p.window, p.chunk, p.max_len);
+  const SeqRange r = seq_range(__builtin_amdgcn_readfirstlane(p.lens[b]), p.cap, p.window, p.max_len);
   if (chunk_id >= r.nchunks) return;
   // position held by slot s is s + pos_base, or cap less when that would lie beyond the last one
   const int pos_base = (r.len > 0) ? ((r.len - 1) / p.cap) * p.cap : 0;
@@ -81,14 +88,15 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
     int pp = s + pos_base;
     return (pp > r.len - 1) ? pp - p.cap : pp;   // negative for a slot that was never written
   };
-  const int c0 = r.s_begin + chunk_id * p.chunk;
-  const int c1 = min(r.s_end, c0 + p.chunk);
+  const int c0 = r.s_begin + chunk_id * r.chunk;
+  const int c1 = min(r.s_end, c0 + r.chunk);
   const int n = lane & 15, c = lane >> 4;
   const int G = p.G;
   const int head = g * G + min(n, G - 1);
 
-  const bf16_t *kbase = p.kc + ((size_t)(b * p.n_kv + g) * p.cap) * D;
-  const bf16_t *vbase = p.vc + ((size_t)(b * p.n_kv + g) * p.cap) * D;
+  const int seq = (p.rows_per_seq > 1) ? b / p.rows_per_seq : b;
+  const bf16_t *kbase = p.kc + ((size_t)(seq * p.n_kv + g) * p.cap) * D;
+  const bf16_t *vbase = p.vc + ((size_t)(seq * p.n_kv + g) * p.cap) * D;
   // lane's K bytes for slot block `blk`: slot blk + tb*16 + n, d chunk c*KS*8 .. +KS*8
   const size_t k_lane = (size_t)n * D + c * KS * 8;
   const size_t v_lane = (size_t)lane * 8;
@@ -286,7 +294,7 @@ __global__ __launch_bounds__(256) void attn_reduce_kernel(AttnParams p) {
   const int d4 = (threadIdx.x % TPP) * 4;
   if (pair >= p.B * p.n_q) return;
   const int b = pair / p.n_q, hq = pair - b * p.n_q;
-  const SeqRange r = seq_range(p.lens[b], p.cap, p.window, p.chunk, p.max_len);
+  const SeqRange r = seq_range(p.lens[b], p.cap, p.window, p.max_len);
   if (r.nchunks <= 1) return;  // already finished by the first kernel
   const float sink2 = p.sinks ? p.sinks[hq] * 1.4426950408889634f : -INFINITY;
   const size_t slot0 = (size_t)b * p.max_chunks * p.n_q + hq;
@@ -353,18 +361,18 @@ __global__ __launch_bounds__(256) void kv_cache_write_kernel(bf16_t *__restrict_
   }
 }
 
-static int attn_chunk_tokens(int span) { return span > 1024 ? 512 : 256; }
-
 struct AttnPlan {
-  int chunk, max_chunks;
+  int max_chunks;
   size_t part_o_bytes, part_ml_bytes;
 };
 
 static AttnPlan attn_plan(int B, int n_q, int D, int max_len) {
   AttnPlan pl;
-  pl.chunk = attn_chunk_tokens(max_len);
-  // a window range can start up to 63 slots before its first active position
-  pl.max_chunks = (max_len + ATT_BLOCK - 1 + pl.chunk - 1) / pl.chunk;
+  // most work items any row can have: rows choose their chunk length from their own slot range,
+  // which can start up to 63 slots before the first active position
+  const int longest = max_len + ATT_BLOCK - 1;
+  pl.max_chunks = (longest + attn_chunk_tokens(longest) - 1) / attn_chunk_tokens(longest);
+  if (longest > 1024) pl.max_chunks = std::max(pl.max_chunks, (1024 + 255) / 256);
   if (pl.max_chunks < 1) pl.max_chunks = 1;
   pl.part_o_bytes = align_up((size_t)B * pl.max_chunks * n_q * D * sizeof(float), 256);
   pl.part_ml_bytes = align_up((size_t)B * pl.max_chunks * n_q * 2 * sizeof(float), 256);
@@ -407,10 +415,11 @@ extern "C" size_t gptoss_attn_workspace_bytes(int B, int n_q, int n_kv, int head
          align_up((size_t)B * max_chunks * n_q * 2 * sizeof(float), 256);
 }
 
-extern "C" int gptoss_attn_decode(const float *q, const void *k_cache, const void *v_cache,
-                                  const int *lens, const float *sinks, void *out, int B, int n_q,
-                                  int n_kv, int head_dim, int capacity, int window, int max_len,
-                                  void *workspace, size_t workspace_bytes, void *stream) {
+// B query rows; row b reads the cache of sequence b / rows_per_seq up to its own lens[b]
+static int attn_launch(const float *q, const void *k_cache, const void *v_cache, const int *lens,
+                       const float *sinks, void *out, int B, int rows_per_seq, int n_q, int n_kv,
+                       int head_dim, int capacity, int window, int max_len, void *workspace,
+                       size_t workspace_bytes, void *stream) {
   GPTOSS_REQUIRE(q && k_cache && v_cache && lens && out, GPTOSS_ERR_NULL, "attn_decode: null pointer");
   GPTOSS_REQUIRE(B > 0 && n_q > 0 && n_kv > 0 && n_q % n_kv == 0 && n_q / n_kv <= 16, GPTOSS_ERR_DIM,
                  "attn_decode: need n_q %% n_kv == 0 and n_q/n_kv <= 16 (n_q=%d n_kv=%d)", n_q, n_kv);
@@ -441,12 +450,12 @@ extern "C" int gptoss_attn_decode(const float *q, const void *k_cache, const voi
   p.part_o = (float *)workspace;
   p.part_ml = (float *)((unsigned char *)workspace + pl.part_o_bytes);
   p.B = B;
+  p.rows_per_seq = rows_per_seq;
   p.n_q = n_q;
   p.n_kv = n_kv;
   p.G = n_q / n_kv;
   p.cap = capacity;
   p.window = window;
-  p.chunk = pl.chunk;
   p.max_chunks = pl.max_chunks;
   p.max_len = max_len;
   p.scale_log2e = 1.4426950408889634f / sqrtf((float)head_dim);
@@ -468,4 +477,45 @@ extern "C" int gptoss_attn_decode(const float *q, const void *k_cache, const voi
     GPTOSS_LAUNCH_CHECK("attn_reduce_kernel");
   }
   return GPTOSS_OK;
+}
+
+extern "C" int gptoss_attn_decode(const float *q, const void *k_cache, const void *v_cache,
+                                  const int *lens, const float *sinks, void *out, int B, int n_q,
+                                  int n_kv, int head_dim, int capacity, int window, int max_len,
+                                  void *workspace, size_t workspace_bytes, void *stream) {
+  return attn_launch(q, k_cache, v_cache, lens, sinks, out, B, 1, n_q, n_kv, head_dim, capacity, window,
+                     max_len, workspace, workspace_bytes, stream);
+}
+
+__global__ __launch_bounds__(256) void prefill_lens_kernel(int *lens, int rows, int T, int pos0) {
+  const int r = blockIdx.x * 256 + threadIdx.x;
+  if (r < rows) lens[r] = pos0 + r % T + 1;
+}
+
+extern "C" size_t gptoss_attn_prefill_workspace_bytes(int B, int T, int n_q, int n_kv, int head_dim,
+                                                      int max_len) {
+  if (B <= 0 || T <= 0) return 0;
+  size_t rows = (size_t)B * T;
+  if (rows > 0x7fffffff) return 0;
+  return align_up(rows * sizeof(int), 256) + gptoss_attn_workspace_bytes((int)rows, n_q, n_kv, head_dim, max_len);
+}
+
+extern "C" int gptoss_attn_prefill(const float *q, const void *k_cache, const void *v_cache,
+                                   const float *sinks, void *out, int B, int T, int pos0, int n_q,
+                                   int n_kv, int head_dim, int capacity, int window, void *workspace,
+                                   size_t workspace_bytes, void *stream) {
+  GPTOSS_REQUIRE(B > 0 && T > 0 && pos0 >= 0 && (long long)B * T < (1ll << 24), GPTOSS_ERR_DIM,
+                 "attn_prefill: need B > 0, T > 0, pos0 >= 0 and B*T < 2^24 (B=%d T=%d)", B, T);
+  GPTOSS_REQUIRE(window == 0 || pos0 + T <= capacity, GPTOSS_ERR_DIM,
+                 "attn_prefill: a windowed cache must hold all %d positions (capacity=%d): rows of one "
+                 "launch read the cache as it is after the last position was written", pos0 + T, capacity);
+  const int rows = B * T;
+  const size_t lens_bytes = align_up((size_t)rows * sizeof(int), 256);
+  GPTOSS_REQUIRE(workspace && aligned(workspace, 256) && workspace_bytes > lens_bytes, GPTOSS_ERR_WORKSPACE,
+                 "attn_prefill: workspace missing, misaligned or too small");
+  int *lens = (int *)workspace;
+  prefill_lens_kernel<<<(rows + 255) / 256, 256, 0, (hipStream_t)stream>>>(lens, rows, T, pos0);
+  GPTOSS_LAUNCH_CHECK("prefill_lens_kernel");
+  return attn_launch(q, k_cache, v_cache, lens, sinks, out, rows, T, n_q, n_kv, head_dim, capacity, window,
+                     pos0 + T, (unsigned char *)workspace + lens_bytes, workspace_bytes - lens_bytes, stream);
 }

@@ -61,6 +61,17 @@ struct gptoss_engine {
   void *moe_ws, *attn_ws;
   size_t moe_ws_bytes, attn_ws_bytes;
   size_t device_bytes;
+  // prompt processing (many positions of a sequence at once): activations for up to pf.rows rows,
+  // and a linear K/V scratch for the sliding-window layers when a prompt is longer than their ring
+  struct Prefill {
+    int rows;  // 0: not available
+    int *tokens;
+    float *x, *qkv, *q, *tb2;
+    bf16_t *t, *attn_out, *k_scratch, *v_scratch;
+    size_t scratch_tokens;  // positions (summed over sequences) the scratch holds
+    void *moe_ws, *attn_ws;
+    size_t moe_ws_bytes, attn_ws_bytes;
+  } pf;
   // fp32-faithful mode (GPTOSS_ENGINE_PRECISE): the .bin payload as it is, fp32 KV caches and
   // fp32 intermediates
   struct Precise {
@@ -214,8 +225,12 @@ int dense_gemm(const bf16_t *A, const bf16_t *W, const float *bias, void *out, i
       break;
     }
   if (B > 96) rpt = (g.n_col_tiles >= 64) ? 128 : 96;
+  if (B >= 2048) rpt = 160;  // a prompt pass: thousands of rows, every weight fragment feeds five MFMAs
   return run_gemm(g, false, epi, rpt, cdiv(B, rpt), s);
 }
+
+// most rows (sequences x positions) one prompt-processing pass works on
+constexpr long long PREFILL_ROWS = 8192;
 
 void destroy(gptoss_engine *e) {
   if (!e) return;
@@ -374,6 +389,7 @@ extern "C" int gptoss_engine_create(const gptoss_config *cfg, const float *host_
   e->device_bytes = 0;
   e->h_tokens = e->h_next = nullptr;
   e->stream = nullptr;
+  e->pf.rows = 0;
   Builder b;
   b.e = e;
   b.hip(hipStreamCreate(&e->stream), "hipStreamCreate");
@@ -522,6 +538,35 @@ extern "C" int gptoss_engine_create(const gptoss_config *cfg, const float *host_
   e->moe_ws = b.alloc<unsigned char>(e->moe_ws_bytes);
   e->attn_ws_bytes = std::max<size_t>(256, gptoss_attn_workspace_bytes(B, nq, nkv, D, max_seq));
   e->attn_ws = b.alloc<unsigned char>(e->attn_ws_bytes);
+  if (!(flags & GPTOSS_ENGINE_NO_PREFILL)) {
+    gptoss_engine::Prefill &pf = e->pf;
+    const int R = (int)std::min<long long>((long long)max_batch * max_seq, PREFILL_ROWS);
+    pf.tokens = b.alloc<int>(R);
+    pf.x = b.alloc<float>((size_t)R * H);
+    pf.t = b.alloc<bf16_t>((size_t)R * H);
+    pf.qkv = b.alloc<float>((size_t)R * qkv_dim);
+    pf.q = b.alloc<float>((size_t)R * nq * D);
+    pf.attn_out = b.alloc<bf16_t>((size_t)R * nq * D);
+    pf.tb2 = b.alloc<float>((size_t)R * H);
+    pf.moe_ws_bytes = gptoss_moe_workspace_bytes(R, E, k, H, I);
+    pf.moe_ws = b.alloc<unsigned char>(pf.moe_ws_bytes);
+    // rows of one launch: B sequences x T positions with B*T <= R and T <= max_seq
+    pf.attn_ws_bytes = gptoss_attn_prefill_workspace_bytes(1, R, nq, nkv, D, std::min(R, max_seq));
+    pf.attn_ws = b.alloc<unsigned char>(pf.attn_ws_bytes);
+    pf.k_scratch = pf.v_scratch = nullptr;
+    pf.scratch_tokens = 0;
+    if (W > 0 && max_seq > (int)align_up((size_t)W, 64)) {
+      pf.scratch_tokens = (size_t)R + (size_t)64 * max_batch;
+      pf.k_scratch = b.alloc<bf16_t>(pf.scratch_tokens * nkv * D);
+      pf.v_scratch = b.alloc<bf16_t>(pf.scratch_tokens * nkv * D);
+      // slots past a prompt's end are masked, but must hold finite values
+      if (b.ok()) {
+        b.hip(hipMemsetAsync(pf.k_scratch, 0, pf.scratch_tokens * nkv * D * sizeof(bf16_t), e->stream), "memset");
+        b.hip(hipMemsetAsync(pf.v_scratch, 0, pf.scratch_tokens * nkv * D * sizeof(bf16_t), e->stream), "memset");
+      }
+    }
+    if (b.ok()) pf.rows = R;
+  }
   if (b.ok()) b.hip(hipStreamSynchronize(e->stream), "sync");
   if (!b.ok()) {
     destroy(e);
@@ -606,6 +651,99 @@ extern "C" int gptoss_engine_step(gptoss_engine *e, const int *host_tokens, int 
   return GPTOSS_OK;
 }
 
+// Positions 0..T-1 of sequences seq0..seq0+Bc-1 in one pass (Bc*T <= pf.rows): same kernels and the
+// same per-row arithmetic as T lock-step steps, so the caches and the arg-max after the last
+// position are those the lock-step loop would have produced (bit for bit as long as no sliding
+// window ring has wrapped; after that the window layers sum their scores in another order).
+static int prefill_chunk(gptoss_engine *e, const int *host_tokens, int seq0, int Bc, int T) {
+  const gptoss_config &c = e->cfg;
+  const int H = c.hidden_dim, V = c.vocab_size, L = c.n_layers, E = c.n_experts, k = c.experts_per_token;
+  const int D = c.head_dim, nq = c.n_attn_heads, nkv = c.n_kv_heads, I = c.intermediate_dim;
+  const int qkv_dim = (nq + 2 * nkv) * D;
+  const int rows = Bc * T;
+  gptoss_engine::Prefill &pf = e->pf;
+  hipStream_t s = e->stream;
+  int rc;
+#define STEP(call)                   \
+  do {                               \
+    rc = (call);                     \
+    if (rc != GPTOSS_OK) return rc;  \
+  } while (0)
+  GPTOSS_HIP(hipMemcpyAsync(pf.tokens, host_tokens, sizeof(int) * rows, hipMemcpyHostToDevice, s));
+  STEP(run_embedding(e->embedding, pf.tokens, pf.x, rows, H, V, s));
+  for (int l = 0; l < L; l++) {
+    const LayerWeights &w = e->layers[l];
+    if (l == 0) STEP(run_rmsnorm(pf.x, nullptr, w.attn_norm, pf.t, nullptr, rows, H, s));
+    STEP(dense_gemm(pf.t, w.w_qkv, w.b_qkv, pf.qkv, EPI_F32, rows, qkv_dim, H, s));
+    const size_t seq_elems = (size_t)nkv * w.cache_cap * D;
+    bf16_t *kc = w.k_cache + seq_elems * seq0, *vc = w.v_cache + seq_elems * seq0;
+    if (T > w.cache_cap) {
+      // a sliding-window ring shorter than the prompt: attention reads a linear copy of the
+      // prompt's K/V, the ring receives the positions it would hold after T lock-step steps
+      const int cap_t = (int)align_up((size_t)T, 64);
+      STEP(run_rope_store_rows(pf.qkv, pf.q, pf.k_scratch, pf.v_scratch, e->cos_t, e->sin_t, rows, T, nq, nkv, D,
+                               cap_t, 0, 0, s));
+      STEP(run_rope_store_rows(pf.qkv, nullptr, kc, vc, e->cos_t, e->sin_t, rows, T, nq, nkv, D, w.cache_cap, 0,
+                               T - w.cache_cap, s));
+      STEP(gptoss_attn_prefill(pf.q, pf.k_scratch, pf.v_scratch, w.sinks, pf.attn_out, Bc, T, 0, nq, nkv, D, cap_t,
+                               w.window, pf.attn_ws, pf.attn_ws_bytes, s));
+    } else {
+      STEP(run_rope_store_rows(pf.qkv, pf.q, kc, vc, e->cos_t, e->sin_t, rows, T, nq, nkv, D, w.cache_cap, 0, 0, s));
+      STEP(gptoss_attn_prefill(pf.q, kc, vc, w.sinks, pf.attn_out, Bc, T, 0, nq, nkv, D, w.cache_cap, w.window,
+                               pf.attn_ws, pf.attn_ws_bytes, s));
+    }
+    STEP(dense_gemm(pf.attn_out, w.w_o, w.b_o, pf.tb2, EPI_F32, rows, H, nq * D, s));
+    STEP(run_rmsnorm(pf.x, pf.tb2, w.mlp_norm, pf.t, nullptr, rows, H, s));
+    gptoss_moe_weights mw;
+    mw.n_experts = E;
+    mw.top_k = k;
+    mw.hidden = H;
+    mw.intermediate = I;
+    mw.swiglu_limit = c.swiglu_limit;
+    mw.w_router = w.w_router;
+    mw.b_router = w.b_router;
+    mw.w1 = w.w1;
+    mw.b1 = w.b1;
+    mw.w2 = w.w2;
+    mw.b2 = w.b2;
+    STEP(gptoss_moe_forward(&mw, pf.t, rows, pf.x, 1, pf.moe_ws, pf.moe_ws_bytes, s));
+    if (l + 1 < L) STEP(run_rmsnorm(pf.x, nullptr, e->layers[l + 1].attn_norm, pf.t, nullptr, rows, H, s));
+  }
+  // only the last position of every sequence goes through the final norm and the classifier
+  STEP(run_gather_rows(pf.x, e->x, Bc, H, T, T - 1, s));
+  STEP(run_rmsnorm(e->x, nullptr, e->final_norm, e->t, nullptr, Bc, H, s));
+  if (e->logits) {
+    STEP(dense_gemm(e->t, e->unembedding, nullptr, e->logits + (size_t)seq0 * V, EPI_F32, Bc, V, H, s));
+    STEP(run_argmax(e->logits + (size_t)seq0 * V, e->d_next + seq0, Bc, V, s));
+  } else {
+    STEP(dense_gemm(e->t, e->unembedding, nullptr, nullptr, EPI_ARGMAX, Bc, V, H, s, e->amax_val, e->amax_idx));
+    STEP(run_argmax_tiles(e->amax_val, e->amax_idx, e->d_next + seq0, Bc, gemm_col_tiles(V), s));
+  }
+#undef STEP
+  return GPTOSS_OK;
+}
+
+extern "C" int gptoss_engine_prefill(gptoss_engine *e, const int *host_tokens, int B, int T, int *host_next) {
+  GPTOSS_REQUIRE(e && host_tokens && host_next, GPTOSS_ERR_NULL, "engine_prefill: null pointer");
+  GPTOSS_REQUIRE(!(e->flags & GPTOSS_ENGINE_PRECISE) && e->pf.rows > 0, GPTOSS_ERR_STATE,
+                 "engine_prefill: not available (GPTOSS_ENGINE_PRECISE or GPTOSS_ENGINE_NO_PREFILL)");
+  GPTOSS_REQUIRE(B >= 1 && B <= e->max_batch, GPTOSS_ERR_DIM, "engine_prefill: batch %d outside 1..%d", B, e->max_batch);
+  GPTOSS_REQUIRE(T >= 1 && T <= e->max_seq && T <= e->pf.rows, GPTOSS_ERR_DIM,
+                 "engine_prefill: %d positions outside 1..%d", T, std::min(e->max_seq, e->pf.rows));
+  const int per = std::max(1, e->pf.rows / T);  // sequences per pass
+  for (int s0 = 0; s0 < B; s0 += per) {
+    const int bc = std::min(per, B - s0);
+    int rc = prefill_chunk(e, host_tokens + (size_t)s0 * T, s0, bc, T);
+    if (rc != GPTOSS_OK) return rc;
+    // the token staging buffer and the activations are reused by the next pass
+    GPTOSS_HIP(hipStreamSynchronize(e->stream));
+  }
+  GPTOSS_HIP(hipMemcpyAsync(e->h_next, e->d_next, sizeof(int) * B, hipMemcpyDeviceToHost, e->stream));
+  GPTOSS_HIP(hipStreamSynchronize(e->stream));
+  memcpy(host_next, e->h_next, sizeof(int) * B);
+  return GPTOSS_OK;
+}
+
 extern "C" int gptoss_engine_generate(gptoss_engine *e, const int *host_prompts, const int *host_n_prompt,
                                       int prompt_stride, int n_req, int max_seq_len, int *host_out,
                                       long long *n_generated) {
@@ -625,9 +763,35 @@ extern "C" int gptoss_engine_generate(gptoss_engine *e, const int *host_prompts,
     std::vector<char> active(B, 1);
     int active_count = B;
     for (int i = 0; i < B; i++) cur_tok[i] = host_prompts[(size_t)(r0 + i) * prompt_stride];
-    for (int pos = 0; pos < max_seq_len - 1 && active_count > 0; pos++) {
-      int rc = gptoss_engine_step(e, cur_tok.data(), pos, B, next.data());
-      if (rc != GPTOSS_OK) return rc;
+    // The prompt positions every sequence of the batch has in common go through one prefill pass
+    // instead of one lock-step step each (the reference feeds prompts token by token,
+    // getp_run_submit.cpp:60-72).  The pass stops before a prompt's own stop token, which ends
+    // that sequence in the lock-step loop, and before the last position the loop may visit.
+    int first_pos = 0;
+    if (e->pf.rows > 0 && !(e->flags & GPTOSS_ENGINE_PRECISE)) {
+      int T = std::min(max_seq_len - 1, e->pf.rows);
+      for (int i = 0; i < B; i++) {
+        const int *pt = host_prompts + (size_t)(r0 + i) * prompt_stride;
+        const int np = host_n_prompt[r0 + i];
+        T = std::min(T, np);
+        for (int j = 1; j < T; j++)
+          if (pt[j] == 199999 || pt[j] == 200002) T = j;
+      }
+      if (T >= 2) {
+        std::vector<int> toks((size_t)B * T);
+        for (int i = 0; i < B; i++)
+          memcpy(&toks[(size_t)i * T], host_prompts + (size_t)(r0 + i) * prompt_stride, sizeof(int) * T);
+        int rc = gptoss_engine_prefill(e, toks.data(), B, T, next.data());
+        if (rc != GPTOSS_OK) return rc;
+        first_pos = T;
+        for (int i = 0; i < B; i++) cur_pos[i] = T - 1;  // the loop body below finishes position T-1
+      }
+    }
+    for (int pos = first_pos > 0 ? first_pos - 1 : 0; pos < max_seq_len - 1 && active_count > 0; pos++) {
+      if (pos >= first_pos) {
+        int rc = gptoss_engine_step(e, cur_tok.data(), pos, B, next.data());
+        if (rc != GPTOSS_OK) return rc;
+      }
       for (int i = 0; i < B; i++) {
         if (!active[i]) continue;
         const int *pt = host_prompts + (size_t)(r0 + i) * prompt_stride;

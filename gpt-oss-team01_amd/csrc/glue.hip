@@ -62,20 +62,27 @@ __global__ __launch_bounds__(256) void rope_store_kernel(const float *__restrict
                                                          bf16_t *__restrict__ kc, bf16_t *__restrict__ vc,
                                                          const float *__restrict__ cos_t,
                                                          const float *__restrict__ sin_t, int n_q,
-                                                         int n_kv, int D, int cap, int pos) {
-  const int b = blockIdx.x;
+                                                         int n_kv, int D, int cap, int pos0, int T,
+                                                         int store_from) {
+  // row r of the batch is position pos0 + r % T of sequence r / T (T = 1: one lock-step position)
+  const int r = blockIdx.x;
+  const int b = r / T;
+  const int pos = pos0 + (r - b * T);
   const int half = D >> 1;
   const int q_dim = n_q * D, kv_dim = n_kv * D;
-  const float *row = qkv + (size_t)b * (q_dim + 2 * kv_dim);
+  const float *row = qkv + (size_t)r * (q_dim + 2 * kv_dim);
   const float *cs = cos_t + (size_t)pos * half, *sn = sin_t + (size_t)pos * half;
   const int slot = pos % cap;
-  for (int p = threadIdx.x; p < n_q * half; p += 256) {
-    int h = p / half, j = p - h * half;
-    float x1 = row[h * D + j], x2 = row[h * D + half + j];
-    float c = cs[j], s = sn[j];
-    q_out[(size_t)b * q_dim + h * D + j] = __fsub_rn(__fmul_rn(x1, c), __fmul_rn(x2, s));
-    q_out[(size_t)b * q_dim + h * D + half + j] = __fadd_rn(__fmul_rn(x2, c), __fmul_rn(x1, s));
+  if (q_out != nullptr) {
+    for (int p = threadIdx.x; p < n_q * half; p += 256) {
+      int h = p / half, j = p - h * half;
+      float x1 = row[h * D + j], x2 = row[h * D + half + j];
+      float c = cs[j], s = sn[j];
+      q_out[(size_t)r * q_dim + h * D + j] = __fsub_rn(__fmul_rn(x1, c), __fmul_rn(x2, s));
+      q_out[(size_t)r * q_dim + h * D + half + j] = __fadd_rn(__fmul_rn(x2, c), __fmul_rn(x1, s));
+    }
   }
+  if (pos < store_from) return;  // a ring cache keeps only the last positions of a prefill
   for (int p = threadIdx.x; p < n_kv * half; p += 256) {
     int g = p / half, j = p - g * half;
     float x1 = row[q_dim + g * D + j], x2 = row[q_dim + g * D + half + j];
@@ -192,11 +199,34 @@ int run_rmsnorm(float *x, const float *residual, const float *weight, bf16_t *t_
   return GPTOSS_OK;
 }
 
+// dst[i, :] = src[(i * stride + offset), :], n floats per row (n % 4 == 0)
+__global__ __launch_bounds__(256) void gather_rows_kernel(const float *__restrict__ src,
+                                                          float *__restrict__ dst, int n, int stride,
+                                                          int offset) {
+  const float *sp = src + ((size_t)blockIdx.x * stride + offset) * n;
+  float *dp = dst + (size_t)blockIdx.x * n;
+  for (int i = threadIdx.x * 4; i < n; i += 256 * 4)
+    *reinterpret_cast<f32x4 *>(dp + i) = *reinterpret_cast<const f32x4 *>(sp + i);
+}
+
+int run_gather_rows(const float *src, float *dst, int rows, int n, int stride, int offset, hipStream_t s) {
+  gather_rows_kernel<<<rows, 256, 0, s>>>(src, dst, n, stride, offset);
+  GPTOSS_LAUNCH_CHECK("gather_rows_kernel");
+  return GPTOSS_OK;
+}
+
 int run_rope_store(const float *qkv, float *q_out, bf16_t *kc, bf16_t *vc, const float *cos_t,
                    const float *sin_t, int B, int n_q, int n_kv, int D, int cap, int pos,
                    hipStream_t s) {
+  return run_rope_store_rows(qkv, q_out, kc, vc, cos_t, sin_t, B, 1, n_q, n_kv, D, cap, pos, 0, s);
+}
+
+int run_rope_store_rows(const float *qkv, float *q_out, bf16_t *kc, bf16_t *vc, const float *cos_t,
+                        const float *sin_t, int rows, int T, int n_q, int n_kv, int D, int cap, int pos0,
+                        int store_from, hipStream_t s) {
   TraceScope ts("rope_store", s);
-  rope_store_kernel<<<B, 256, 0, s>>>(qkv, q_out, kc, vc, cos_t, sin_t, n_q, n_kv, D, cap, pos);
+  rope_store_kernel<<<rows, 256, 0, s>>>(qkv, q_out, kc, vc, cos_t, sin_t, n_q, n_kv, D, cap, pos0, T,
+                                         store_from);
   GPTOSS_LAUNCH_CHECK("rope_store_kernel");
   return GPTOSS_OK;
 }

@@ -11,6 +11,13 @@ int run_rmsnorm(float *x, const float *residual, const float *weight, bf16_t *t_
 int run_rope_store(const float *qkv, float *q_out, bf16_t *kc, bf16_t *vc, const float *cos_t,
                    const float *sin_t, int B, int n_q, int n_kv, int D, int cap, int pos,
                    hipStream_t s);
+// rows = sequences * T: row r is position pos0 + r % T of sequence r / T; K/V of positions below
+// store_from are not stored; q_out may be null
+int run_rope_store_rows(const float *qkv, float *q_out, bf16_t *kc, bf16_t *vc, const float *cos_t,
+                        const float *sin_t, int rows, int T, int n_q, int n_kv, int D, int cap, int pos0,
+                        int store_from, hipStream_t s);
+// dst[i, :] = src[i * stride + offset, :]
+int run_gather_rows(const float *src, float *dst, int rows, int n, int stride, int offset, hipStream_t s);
 int run_argmax(const float *logits, int *ids, int B, int V, hipStream_t s);
 int run_argmax_tiles(const float *val, const int *idx, int *ids, int B, int n_tiles, hipStream_t s);
 int run_f32_to_bf16(const float *src, bf16_t *dst, size_t n, hipStream_t s);

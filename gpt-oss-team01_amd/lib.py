@@ -20,6 +20,7 @@ PACK_GLU = 2
 ENGINE_SYNTHETIC = 1
 ENGINE_PRECISE = 2
 ENGINE_LOGITS = 4
+ENGINE_NO_PREFILL = 8
 
 
 class GptossError(RuntimeError):
@@ -76,6 +77,9 @@ SIGNATURES = {
     "gptoss_engine_create": (_i, [C.POINTER(Config), _vp, _i, _i, _i, C.c_uint64,
                                   C.POINTER(_vp)]),
     "gptoss_engine_step": (_i, [_vp, _vp, _i, _i, _vp]),
+    "gptoss_engine_prefill": (_i, [_vp, _vp, _i, _i, _vp]),
+    "gptoss_attn_prefill_workspace_bytes": (_sz, [_i, _i, _i, _i, _i, _i]),
+    "gptoss_attn_prefill": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _sz, _vp]),
     "gptoss_engine_generate": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp, C.POINTER(C.c_longlong)]),
     "gptoss_engine_destroy": (None, [_vp]),
     "gptoss_engine_debug_views": (_i, [_vp, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_sz)]),

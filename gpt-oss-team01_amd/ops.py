@@ -178,6 +178,27 @@ class AttnDecode:
         return out
 
 
+class AttnPrefill:
+    """The decode attention for T consecutive positions of every sequence at once:
+    q [B,T,n_q,D] fp32 -> out [B,T,n_q,D] bf16; row (b,t) sees cached positions <= pos0 + t."""
+
+    def __init__(self, B, T, n_q, n_kv, head_dim, max_len, device="cuda"):
+        _need_gpu()
+        self.L = _l.load()
+        self.n_q, self.n_kv, self.D = n_q, n_kv, head_dim
+        self.ws_bytes = self.L.gptoss_attn_prefill_workspace_bytes(B, T, n_q, n_kv, head_dim, max_len)
+        self.ws = torch.empty(max(self.ws_bytes, 256), dtype=torch.uint8, device=device)
+
+    def forward(self, q, cache: KVCache, pos0=0, sinks=None, window=0):
+        B, T = q.shape[:2]
+        assert q.dtype == torch.float32 and q.is_contiguous()
+        out = torch.empty(B, T, self.n_q, self.D, dtype=torch.bfloat16, device=q.device)
+        _l.check(self.L.gptoss_attn_prefill(_ptr(q), _ptr(cache.k), _ptr(cache.v), _ptr(sinks), _ptr(out),
+                                            B, T, pos0, self.n_q, self.n_kv, self.D, cache.cap, window,
+                                            _ptr(self.ws), self.ws_bytes, _stream()))
+        return out
+
+
 class KernelTrace:
     """Per-kernel HIP-event timing of the entry points called inside the ``with`` block
     (events are recorded on the stream each kernel is launched on)."""
@@ -226,14 +247,14 @@ class Engine:
     """Single-GPU decode engine over a flat ``.bin`` payload (or synthetic on-device weights)."""
 
     def __init__(self, cfg, weights_flat=None, max_batch=8, max_seq=64, synthetic=False,
-                 precise=False, seed=0, keep_logits=True):
+                 precise=False, seed=0, keep_logits=True, prefill=True):
         _need_gpu()
         import numpy as np
         self.L = _l.load()
         self.cfg = cfg
         self.max_batch, self.max_seq = max_batch, max_seq
         flags = (_l.ENGINE_SYNTHETIC if synthetic else 0) | (_l.ENGINE_PRECISE if precise else 0) | \
-            (_l.ENGINE_LOGITS if keep_logits else 0)
+            (_l.ENGINE_LOGITS if keep_logits else 0) | (0 if prefill else _l.ENGINE_NO_PREFILL)
         self._cc = _l.Config.from_config(cfg)
         wp = None
         if not synthetic:
@@ -250,6 +271,16 @@ class Engine:
         nxt = np.empty_like(tok)
         _l.check(self.L.gptoss_engine_step(self._h, tok.ctypes.data_as(C.c_void_p), int(pos),
                                            tok.size, nxt.ctypes.data_as(C.c_void_p)))
+        return nxt
+
+    def prefill(self, tokens):
+        """Positions 0..T-1 of every sequence (tokens int32 [B, T]) in one pass -> next ids [B]."""
+        import numpy as np
+        tok = np.ascontiguousarray(tokens, dtype=np.int32)
+        B, T = tok.shape
+        nxt = np.empty(B, np.int32)
+        _l.check(self.L.gptoss_engine_prefill(self._h, tok.ctypes.data_as(C.c_void_p), B, T,
+                                              nxt.ctypes.data_as(C.c_void_p)))
         return nxt
 
     def generate(self, prompts, max_seq_len, n_prompt=None):

@@ -185,6 +185,19 @@ int gptoss_attn_decode(const float *q, const void *k_cache, const void *v_cache,
                        int capacity, int window, int max_len, void *workspace,
                        size_t workspace_bytes, void *stream);
 
+/* The same attention for T consecutive positions of every sequence at once (prompt processing):
+ * q fp32 [B, T, n_q, D] and out bf16 [B, T, n_q, D]; row (b, t) attends to the cached positions up
+ * to pos0 + t of sequence b, with the arithmetic gptoss_attn_decode uses for lens = pos0 + t + 1,
+ * so its result is the one the T lock-step calls of the reference would give
+ * (getp-csrc/submit/getp_run_submit.cpp:60-72 feeds prompts one position per step).  The cache must
+ * already hold positions [0, pos0 + T) of every sequence, all of them (a sliding-window ring
+ * shorter than pos0 + T is refused: copy the prompt's K/V to a linear cache for this call). */
+size_t gptoss_attn_prefill_workspace_bytes(int B, int T, int n_q, int n_kv, int head_dim, int max_len);
+int gptoss_attn_prefill(const float *q, const void *k_cache, const void *v_cache, const float *sinks,
+                        void *out, int B, int T, int pos0, int n_q, int n_kv, int head_dim,
+                        int capacity, int window, void *workspace, size_t workspace_bytes,
+                        void *stream);
+
 /* ------------------------------------------------------------------ engine ------------------ */
 
 /* The 60-byte header of the flat .bin (reference run.cpp:25-45), same field order. */
@@ -204,10 +217,13 @@ enum {
                                   gptoss_engine_debug_views); without it the classifier GEMM keeps only
                                   each row's arg-max, as max_logits_batched consumes them
                                   (getp-csrc/src/model.cpp:144-148) */
-  GPTOSS_ENGINE_PRECISE = 2    /* the reference CPU model's arithmetic (run.cpp:501-717) instead of the
+  GPTOSS_ENGINE_PRECISE = 2,   /* the reference CPU model's arithmetic (run.cpp:501-717) instead of the
                                   reference GPU path's bf16 staging: fp32 weights, activations and KV
                                   cache, double-accumulated dot products.  Reproduces the CPU model's
                                   greedy ids; slow, needs host_weights, 4x the weight memory */
+  GPTOSS_ENGINE_NO_PREFILL = 8 /* no prompt-processing buffers: gptoss_engine_generate feeds prompts one
+                                  position per step, as the reference does
+                                  (getp-csrc/submit/getp_run_submit.cpp:60-72) */
 };
 
 /* Build device weights (bf16, packed) and run state for up to max_batch sequences of up to
@@ -221,6 +237,15 @@ int gptoss_engine_create(const gptoss_config *cfg, const float *host_weights, in
  * (lowest id wins ties) in host_next[B].  Replaces forward_gpu_20b_batched
  * (getp-csrc/src/model.cpp:6-151).  Synchronises once, to hand the ids back. */
 int gptoss_engine_step(gptoss_engine *e, const int *host_tokens, int pos, int B, int *host_next);
+
+/* Positions 0..T-1 of B sequences in one pass: host_tokens int32 [B, T]; fills the KV caches and
+ * returns in host_next[B] the arg-max ids after position T-1, i.e. what T calls of
+ * gptoss_engine_step with pos = 0..T-1 leave behind (identical ids and caches while no
+ * sliding-window ring has wrapped, equal to rounding after that).  Decoding continues with
+ * gptoss_engine_step at pos = T.  The reference has no such pass: it feeds prompts one position
+ * per step (getp-csrc/submit/getp_run_submit.cpp:60-72).  Needs T <= max_seq and T <= 8192; not
+ * available with GPTOSS_ENGINE_PRECISE or GPTOSS_ENGINE_NO_PREFILL. */
+int gptoss_engine_prefill(gptoss_engine *e, const int *host_tokens, int B, int T, int *host_next);
 
 /* Greedy generation with the reference's getp loop semantics
  * (getp-csrc/submit/getp_run_submit.cpp:60-96): prompts int32 [n_req, prompt_stride] with

@@ -161,3 +161,50 @@ def test_attn_batch_larger_than_one_launch_slice(ops, orc):
     want = orc.attn_decode(q.numpy(), K.float().numpy(), V.float().numpy(), lens, sinks.numpy(), 0)
     mx, mean = rel_errors(got, want)
     assert mx <= TOL_MAX and mean <= TOL_MEAN, (mx, mean)
+
+
+@pytest.mark.parametrize("B,T,pos0,n_q,n_kv,D,window", [
+    (3, 40, 0, 8, 2, 32, 0),          # tiny-model heads, whole prompt from position 0
+    (2, 128, 0, 64, 8, 64, 128),      # 20B heads, the window exactly as long as the prompt
+    (2, 300, 0, 64, 8, 64, 128),      # prompt longer than the window (linear cache)
+    (2, 70, 500, 64, 8, 64, 0),       # a later slice of a long context: two chunks per row
+    (1, 200, 1000, 64, 8, 64, 0),     # rows on both sides of the 1024-position chunk-size change
+])
+def test_attn_prefill_rows_equal_decode_calls(ops, orc, B, T, pos0, n_q, n_kv, D, window):
+    """Prompt attention = the decode attention of every position at once: row (b, t) must equal, bit
+    for bit, the decode call with lens = pos0 + t + 1 on the same cache (whatever else is in the
+    launch), and a sample of rows must match the oracle."""
+    S = pos0 + T
+    g = torch.Generator().manual_seed(S + n_q)
+    q = torch.randn(B, T, n_q, D, generator=g)
+    K = torch.randn(B, S, n_kv, D, generator=g).to(torch.bfloat16)
+    V = torch.randn(B, S, n_kv, D, generator=g).to(torch.bfloat16)
+    sinks = torch.randn(n_q, generator=g)
+    cap = (S + 63) // 64 * 64
+    cache = ops.KVCache(B, n_kv, D, cap)
+    cache.k.view(torch.int16).fill_(0x7FC1)
+    cache.v.view(torch.int16).fill_(0x7FC1)
+    cache.write(K.cuda(), V.cuda(), 0)
+    pre = ops.AttnPrefill(B, T, n_q, n_kv, D, S)
+    got = pre.forward(q.cuda(), cache, pos0=pos0, sinks=sinks.cuda(), window=window)
+    torch.cuda.synchronize()
+    assert torch.isfinite(got.float()).all()
+    dec = ops.AttnDecode(B, n_q, n_kv, D, S)
+    for t in sorted({0, 1, T // 3, T // 2, T - 2, T - 1}):
+        lens = torch.full((B,), pos0 + t + 1, dtype=torch.int32)
+        one = dec.forward(q[:, t].contiguous().cuda(), cache, lens.cuda(), sinks.cuda(), window=window,
+                          max_len=pos0 + t + 1)
+        assert torch.equal(got[:, t], one), t
+        want = orc.attn_decode(q[:, t].numpy(), K.float().numpy(), V.float().numpy(), lens.numpy(), sinks.numpy(),
+                               window)
+        mx, mean = rel_errors(got[:, t].float().cpu().numpy(), want)
+        assert mx <= TOL_MAX and mean <= TOL_MEAN, (t, mx, mean)
+
+
+def test_attn_prefill_refuses_a_wrapped_window_ring(ops):
+    from conftest import load_pkg
+    lib = load_pkg("lib")
+    cache = ops.KVCache(1, 8, 64, 128)
+    pre = ops.AttnPrefill(1, 200, 64, 8, 64, 200)
+    with pytest.raises(lib.GptossError):
+        pre.forward(torch.zeros(1, 200, 64, 64).cuda(), cache, window=128)

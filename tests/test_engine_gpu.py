@@ -191,3 +191,88 @@ def test_fused_argmax_equals_argmax_of_logits(ops, tiny):
         b.last_logits(8)
     a.close()
     b.close()
+
+
+def test_prefill_equals_lockstep_steps(ops, tiny):
+    """One prompt pass over T positions must leave the engine where T lock-step steps leave it:
+    the same next ids, and bit-identical logits on the decode steps that follow (T below the
+    sliding window, so no ring has wrapped)."""
+    fx, cfg, flat = tiny
+    prompts = np.asarray(fx["prompts"], np.int32)
+    gold = np.asarray(fx["expected_ids"], np.int32)
+    seqs = np.concatenate([prompts, gold], axis=1)
+    B, T = 8, 32
+    a = ops.Engine(cfg, flat, max_batch=B, max_seq=64)
+    b = ops.Engine(cfg, flat, max_batch=B, max_seq=64)
+    for pos in range(T):
+        na = a.step(seqs[:, pos], pos)
+    la = a.last_logits(B).copy()
+    nb = b.prefill(seqs[:, :T])
+    assert np.array_equal(na, nb)
+    assert np.array_equal(la, b.last_logits(B))
+    for pos in range(T, T + 12):
+        na, nb = a.step(seqs[:, pos], pos), b.step(seqs[:, pos], pos)
+        assert np.array_equal(na, nb), pos
+        assert np.array_equal(a.last_logits(B), b.last_logits(B)), pos
+    a.close()
+    b.close()
+
+
+def test_prefill_longer_than_the_window_and_in_several_passes(ops, orc, tiny):
+    """200-token prompts: longer than the 128-position ring of the sliding-window layers (they read
+    a linear copy during the pass and keep the last 128 positions), and with 48 sequences more rows
+    (9600) than one pass holds (8192), so the last 8 sequences go through in a second pass.
+    Compared with lock-step steps (equal to rounding: a wrapped ring sums in another order) and,
+    for sequences of both passes, with the fp32 oracle."""
+    fx, cfg, flat = tiny
+    rng = np.random.default_rng(11)
+    B, T, S = 48, 200, 212
+    seqs = rng.integers(0, cfg.vocab_size, size=(B, S)).astype(np.int32)
+    a = ops.Engine(cfg, flat, max_batch=B, max_seq=S)
+    b = ops.Engine(cfg, flat, max_batch=B, max_seq=S)
+    for pos in range(T):
+        na = a.step(seqs[:, pos], pos)
+    nb = b.prefill(seqs[:, :T])
+    lb = b.last_logits(B).copy()
+    mx, _ = rel_errors(lb, a.last_logits(B))
+    assert mx <= 5e-3, mx
+    assert (na == nb).mean() >= 0.9
+    for r in (0, 39, 40, 47):
+        cpu = orc.Model(cfg, flat)
+        for pos in range(T):
+            want = cpu.forward(int(seqs[r, pos]), pos)
+        mx, _ = rel_errors(lb[r], want)
+        assert mx <= 2e-2, (r, mx)
+    # decode steps after the pass, per sequence: equal to bf16 rounding, except where that rounding
+    # moves a near-tie of the router to another expert (a handful of sequence-steps)
+    diffs = []
+    for pos in range(T, S):
+        a.step(seqs[:, pos], pos)
+        b.step(seqs[:, pos], pos)
+        la, lb = a.last_logits(B), b.last_logits(B)
+        diffs.append(np.abs(lb - la).max(axis=1) / np.abs(la).max(axis=1))
+    diffs = np.concatenate(diffs)
+    print("prefill vs lock-step after a wrapped window: median", float(np.median(diffs)),
+          "sequence-steps above 5e-3:", int((diffs > 5e-3).sum()), "of", diffs.size)
+    assert np.median(diffs) <= 5e-3
+    assert (diffs > 5e-3).mean() <= 0.03
+    a.close()
+    b.close()
+
+
+def test_generate_with_prefill_equals_generate_without(ops, tiny):
+    """gptoss_engine_generate sends the prompt positions all sequences of a batch share through one
+    pass; its output must be the lock-step loop's, ragged prompt lengths included."""
+    fx, cfg, flat = tiny
+    prompts = np.asarray(fx["prompts"], np.int32)
+    ragged = np.asarray([32, 20, 32, 9, 32, 32, 2, 32], np.int32)   # shared prefixes of 9 and of 2
+    outs = []
+    for prefill in (True, False):
+        eng = ops.Engine(cfg, flat, max_batch=4, max_seq=fx["max_seq_len"], prefill=prefill)
+        outs.append(eng.generate(prompts, fx["max_seq_len"], n_prompt=ragged))
+        outs.append(eng.generate(prompts, fx["max_seq_len"]))          # all 32 prompt tokens in one pass
+        eng.close()
+    assert np.array_equal(outs[0][0], outs[2][0]) and outs[0][1] == outs[2][1]
+    assert np.array_equal(outs[1][0], outs[3][0]) and outs[1][1] == outs[3][1]
+    with pytest.raises(Exception):
+        ops.Engine(cfg, flat, max_batch=2, max_seq=16, prefill=False).prefill(prompts[:2, :8])
