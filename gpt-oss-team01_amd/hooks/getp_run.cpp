@@ -43,7 +43,9 @@ void warm_up(Transformer *transformer, Tokenizer *tokenizer) {
   g_gptoss_max_seq = cfg.seq_len < 1024 ? cfg.seq_len : 1024;
   // GPTOSS_PRECISE=1: the CPU model's fp32/double arithmetic on the GPU (exact greedy ids, slow)
   const char *precise = getenv("GPTOSS_PRECISE");
-  const int flags = (precise && atoi(precise) != 0) ? GPTOSS_ENGINE_PRECISE : 0;
+  const char *lockstep = getenv("GPTOSS_NO_PREFILL");  // prompts one position per step, as the reference
+  const int flags = ((precise && atoi(precise) != 0) ? GPTOSS_ENGINE_PRECISE : 0) |
+                    ((lockstep && atoi(lockstep) != 0) ? GPTOSS_ENGINE_NO_PREFILL : 0);
   if (gptoss_engine_create(&cfg, weights, max_batch, g_gptoss_max_seq, flags, 0, &g_gptoss_engine) != GPTOSS_OK)
     gptoss_die("engine_create");
 }
