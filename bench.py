@@ -321,6 +321,25 @@ def bench_e2e(ops, torch, n_req=1024, n_prompt=128, n_decode=256):
         eng.prefill(prompts[:64])                      # one pass of 64 x 128 = 8192 rows
     pkern = trace.summary()
     dev_gb = eng.device_bytes() / 1e9
+    # Scheduler: 4096 requests (32-token prompts, length limits U[64, 384]) over the 1024 slots.
+    # Continuous schedule (a finished sequence's slot takes the next request at once) against the
+    # reference's batches of 1024 in lock step until the longest sequence of the batch ends.
+    n_sched = 4 * n_req
+    sp = rng.integers(0, cfg.vocab_size, size=(n_sched, 32), dtype=np.int32)
+    limits = rng.integers(64, n_prompt + n_decode + 1, size=n_sched).astype(np.int32)
+    useful = int((limits - 1).sum())
+    t0 = time.perf_counter()
+    eng.generate(sp, n_prompt + n_decode, max_len=limits)
+    t_cont = time.perf_counter() - t0
+    t0 = time.perf_counter()
+    for b0 in range(0, n_sched, n_req):
+        tok = sp[b0:b0 + n_req, 0].copy()
+        for pos in range(int(limits[b0:b0 + n_req].max()) - 1):
+            tok = eng.step(tok, pos)
+    t_lock = time.perf_counter() - t0
+    sched = {"requests": n_sched, "slots": n_req, "positions": useful,
+             "continuous_tok_s": round(useful / t_cont, 1), "lockstep_batches_tok_s": round(useful / t_lock, 1),
+             "workload": "32-token prompts, total length limits U[64,384]"}
     eng.close()
     return {"decode_tok_s": round(n_req * n_decode / t_decode, 1),
             "decode_ms_per_step": round(t_decode / n_decode * 1e3, 3),
@@ -331,6 +350,7 @@ def bench_e2e(ops, torch, n_req=1024, n_prompt=128, n_decode=256):
             "engine_create_s": round(t_create, 1), "device_gb": round(dev_gb, 1),
             "last_step_kernels_us": {k: [c, round(ms * c * 1e3, 1)] for k, (c, ms) in kern.items()},
             "prefill_pass_8192_rows_kernels_us": {k: [c, round(ms * c * 1e3, 1)] for k, (c, ms) in pkern.items()},
+            "scheduler": sched,
             "config": "24 blocks, hidden 2880, 64q/8kv heads x 64, 32 experts top-4, vocab 201088, "
                       "window 128 on even layers; 1024 seqs x (128 prompt + 256 decoded)"}
 

@@ -53,7 +53,7 @@ struct gptoss_engine {
   float *cos_t, *sin_t;  // [max_seq, D/2]
   // run state
   int *d_tokens, *d_next, *d_lens;
-  int *h_tokens, *h_next;  // pinned
+  int *h_tokens, *h_next, *h_lens;  // pinned
   float *x, *qkv, *q, *tb2, *logits;  // logits == nullptr unless GPTOSS_ENGINE_LOGITS
   float *amax_val;                     // [B, column tiles of the classifier]: fused arg-max partials
   int *amax_idx;
@@ -237,6 +237,7 @@ void destroy(gptoss_engine *e) {
   for (void *p : e->allocs) (void)hipFree(p);
   if (e->h_tokens) (void)hipHostFree(e->h_tokens);
   if (e->h_next) (void)hipHostFree(e->h_next);
+  if (e->h_lens) (void)hipHostFree(e->h_lens);
   if (e->stream) (void)hipStreamDestroy(e->stream);
   delete e;
 }
@@ -387,7 +388,7 @@ extern "C" int gptoss_engine_create(const gptoss_config *cfg, const float *host_
   e->max_seq = max_seq;
   e->flags = flags;
   e->device_bytes = 0;
-  e->h_tokens = e->h_next = nullptr;
+  e->h_tokens = e->h_next = e->h_lens = nullptr;
   e->stream = nullptr;
   e->pf.rows = 0;
   Builder b;
@@ -395,6 +396,7 @@ extern "C" int gptoss_engine_create(const gptoss_config *cfg, const float *host_
   b.hip(hipStreamCreate(&e->stream), "hipStreamCreate");
   b.hip(hipHostMalloc((void **)&e->h_tokens, sizeof(int) * max_batch, hipHostMallocDefault), "hipHostMalloc");
   b.hip(hipHostMalloc((void **)&e->h_next, sizeof(int) * max_batch, hipHostMallocDefault), "hipHostMalloc");
+  b.hip(hipHostMalloc((void **)&e->h_lens, sizeof(int) * max_batch, hipHostMallocDefault), "hipHostMalloc");
   if (precise) {
     int rc = create_precise(e, b, host_weights);
     if (rc != GPTOSS_OK) {
@@ -578,10 +580,10 @@ extern "C" int gptoss_engine_create(const gptoss_config *cfg, const float *host_
 
 extern "C" void gptoss_engine_destroy(gptoss_engine *e) { destroy(e); }
 
-extern "C" int gptoss_engine_step(gptoss_engine *e, const int *host_tokens, int pos, int B, int *host_next) {
-  GPTOSS_REQUIRE(e && host_tokens && host_next, GPTOSS_ERR_NULL, "engine_step: null pointer");
-  GPTOSS_REQUIRE(B >= 1 && B <= e->max_batch, GPTOSS_ERR_DIM, "engine_step: batch %d outside 1..%d", B, e->max_batch);
-  GPTOSS_REQUIRE(pos >= 0 && pos < e->max_seq, GPTOSS_ERR_STATE, "engine_step: position %d outside 0..%d", pos, e->max_seq - 1);
+// One decode step.  host_pos == nullptr: every sequence is at position pos (lock step); else
+// sequence i is at its own position host_pos[i] and pos is their maximum.
+static int step_impl(gptoss_engine *e, const int *host_tokens, int pos, const int *host_pos, int B,
+                     int *host_next) {
   const gptoss_config &c = e->cfg;
   const int H = c.hidden_dim, V = c.vocab_size, L = c.n_layers, E = c.n_experts, k = c.experts_per_token;
   const int D = c.head_dim, nq = c.n_attn_heads, nkv = c.n_kv_heads, I = c.intermediate_dim;
@@ -604,14 +606,23 @@ extern "C" int gptoss_engine_step(gptoss_engine *e, const int *host_tokens, int 
     memcpy(host_next, e->h_next, sizeof(int) * B);
     return GPTOSS_OK;
   }
-  STEP(run_fill_int(e->d_lens, B, pos + 1, s));
+  if (host_pos) {
+    for (int i = 0; i < B; i++) e->h_lens[i] = host_pos[i] + 1;
+    GPTOSS_HIP(hipMemcpyAsync(e->d_lens, e->h_lens, sizeof(int) * B, hipMemcpyHostToDevice, s));
+  } else {
+    STEP(run_fill_int(e->d_lens, B, pos + 1, s));
+  }
   STEP(run_embedding(e->embedding, e->d_tokens, e->x, B, H, V, s));
   for (int l = 0; l < L; l++) {
     const LayerWeights &w = e->layers[l];
     if (l == 0) STEP(run_rmsnorm(e->x, nullptr, w.attn_norm, e->t, nullptr, B, H, s));
     STEP(dense_gemm(e->t, w.w_qkv, w.b_qkv, e->qkv, EPI_F32, B, qkv_dim, H, s));
-    STEP(run_rope_store(e->qkv, e->q, w.k_cache, w.v_cache, e->cos_t, e->sin_t, B, nq, nkv, D,
-                        w.cache_cap, pos, s));
+    if (host_pos)
+      STEP(run_rope_store_lens(e->qkv, e->q, w.k_cache, w.v_cache, e->cos_t, e->sin_t, B, nq, nkv, D,
+                               w.cache_cap, e->d_lens, s));
+    else
+      STEP(run_rope_store(e->qkv, e->q, w.k_cache, w.v_cache, e->cos_t, e->sin_t, B, nq, nkv, D,
+                          w.cache_cap, pos, s));
     STEP(gptoss_attn_decode(e->q, w.k_cache, w.v_cache, e->d_lens, w.sinks, e->attn_out, B, nq, nkv, D,
                             w.cache_cap, w.window, pos + 1, e->attn_ws, e->attn_ws_bytes, s));
     STEP(dense_gemm(e->attn_out, w.w_o, w.b_o, e->tb2, EPI_F32, B, H, nq * D, s));
@@ -649,6 +660,29 @@ extern "C" int gptoss_engine_step(gptoss_engine *e, const int *host_tokens, int 
   memcpy(host_next, e->h_next, sizeof(int) * B);
 #undef STEP
   return GPTOSS_OK;
+}
+
+extern "C" int gptoss_engine_step(gptoss_engine *e, const int *host_tokens, int pos, int B, int *host_next) {
+  GPTOSS_REQUIRE(e && host_tokens && host_next, GPTOSS_ERR_NULL, "engine_step: null pointer");
+  GPTOSS_REQUIRE(B >= 1 && B <= e->max_batch, GPTOSS_ERR_DIM, "engine_step: batch %d outside 1..%d", B, e->max_batch);
+  GPTOSS_REQUIRE(pos >= 0 && pos < e->max_seq, GPTOSS_ERR_STATE, "engine_step: position %d outside 0..%d", pos, e->max_seq - 1);
+  return step_impl(e, host_tokens, pos, nullptr, B, host_next);
+}
+
+extern "C" int gptoss_engine_step_ragged(gptoss_engine *e, const int *host_tokens, const int *host_pos, int B,
+                                         int *host_next) {
+  GPTOSS_REQUIRE(e && host_tokens && host_pos && host_next, GPTOSS_ERR_NULL, "engine_step_ragged: null pointer");
+  GPTOSS_REQUIRE(B >= 1 && B <= e->max_batch, GPTOSS_ERR_DIM, "engine_step_ragged: batch %d outside 1..%d", B,
+                 e->max_batch);
+  GPTOSS_REQUIRE(!(e->flags & GPTOSS_ENGINE_PRECISE), GPTOSS_ERR_STATE,
+                 "engine_step_ragged: not available with GPTOSS_ENGINE_PRECISE");
+  int max_pos = 0;
+  for (int i = 0; i < B; i++) {
+    GPTOSS_REQUIRE(host_pos[i] >= 0 && host_pos[i] < e->max_seq, GPTOSS_ERR_STATE,
+                   "engine_step_ragged: sequence %d at position %d outside 0..%d", i, host_pos[i], e->max_seq - 1);
+    max_pos = std::max(max_pos, host_pos[i]);
+  }
+  return step_impl(e, host_tokens, max_pos, host_pos, B, host_next);
 }
 
 // Positions 0..T-1 of sequences seq0..seq0+Bc-1 in one pass (Bc*T <= pf.rows): same kernels and the
@@ -744,17 +778,12 @@ extern "C" int gptoss_engine_prefill(gptoss_engine *e, const int *host_tokens, i
   return GPTOSS_OK;
 }
 
-extern "C" int gptoss_engine_generate(gptoss_engine *e, const int *host_prompts, const int *host_n_prompt,
-                                      int prompt_stride, int n_req, int max_seq_len, int *host_out,
-                                      long long *n_generated) {
-  GPTOSS_REQUIRE(e && host_prompts && host_n_prompt && host_out, GPTOSS_ERR_NULL, "engine_generate: null pointer");
-  GPTOSS_REQUIRE(n_req >= 0 && prompt_stride >= 1 && max_seq_len >= 1 && max_seq_len <= e->max_seq + 1,
-                 GPTOSS_ERR_DIM, "engine_generate: max_seq_len %d needs an engine with max_seq >= %d",
-                 max_seq_len, max_seq_len - 1);
+// The reference's schedule: requests in batches of max_batch, every batch in lock step until its
+// last sequence ends (getp_run_submit.cpp:13-87).
+static int generate_lockstep(gptoss_engine *e, const int *host_prompts, const int *host_n_prompt,
+                             int prompt_stride, int n_req, int max_seq_len, int *host_out,
+                             long long *n_generated) {
   long long total = 0;
-  for (int r = 0; r < n_req; r++)
-    GPTOSS_REQUIRE(host_n_prompt[r] >= 1 && host_n_prompt[r] <= prompt_stride, GPTOSS_ERR_DIM,
-                   "engine_generate: request %d has %d prompt tokens", r, host_n_prompt[r]);
   // requests are served in batches of max_batch, all sequences of a batch in lock step
   // (getp_run_submit.cpp:13-87)
   for (int r0 = 0; r0 < n_req; r0 += e->max_batch) {
@@ -817,6 +846,129 @@ extern "C" int gptoss_engine_generate(gptoss_engine *e, const int *host_prompts,
   }
   if (n_generated) *n_generated = total;
   return GPTOSS_OK;
+}
+
+// Continuous batching: max_batch slots; a slot whose sequence ended (stop id or its length limit)
+// takes the next waiting request at once, at position 0, while the other slots carry on at their
+// own positions.  Every request sees the arithmetic it would see alone, so its output is the one
+// the lock-step schedule gives; only the order of the work changes.  host_max_len (optional) limits
+// request r to host_max_len[r] positions in all (prompt included) instead of max_seq_len.
+static int generate_continuous(gptoss_engine *e, const int *host_prompts, const int *host_n_prompt,
+                               int prompt_stride, int n_req, int max_seq_len, const int *host_max_len,
+                               int *host_out, long long *n_generated) {
+  long long total = 0;
+  const int B = std::min(e->max_batch, n_req);
+  if (B == 0) {
+    if (n_generated) *n_generated = 0;
+    return GPTOSS_OK;
+  }
+  std::vector<int> req(B, -1), cur_tok(B, 0), cur_pos(B, 0), next(B);
+  int next_req = 0, active_count = 0;
+  auto limit = [&](int r) { return host_max_len ? std::min(host_max_len[r], max_seq_len) : max_seq_len; };
+  auto finish = [&](int i) {
+    const int r = req[i];
+    int generated_len = cur_pos[i] - host_n_prompt[r];
+    if (generated_len < 0) generated_len = 0;
+    host_out[(size_t)r * (max_seq_len + 1) + generated_len + 1] = -1;
+    total += generated_len + 1;
+    req[i] = -1;
+    active_count--;
+  };
+  auto admit = [&](int i) {
+    // requests that may not even take one step are closed as the lock-step loop closes them
+    while (next_req < n_req) {
+      const int r = next_req++;
+      req[i] = r;
+      cur_tok[i] = host_prompts[(size_t)r * prompt_stride];
+      cur_pos[i] = 0;
+      active_count++;
+      if (limit(r) - 1 > 0) return;
+      finish(i);
+    }
+    cur_tok[i] = 0;
+    cur_pos[i] = 0;
+  };
+  for (int i = 0; i < B; i++) admit(i);
+
+  // the prompt positions the first B requests share go through one prompt pass
+  bool first_wave = true;
+  for (int i = 0; i < B; i++) first_wave = first_wave && req[i] == i;
+  int skip_step = 0;
+  if (first_wave && e->pf.rows > 0) {
+    int T = e->pf.rows;
+    for (int i = 0; i < B; i++) {
+      const int *pt = host_prompts + (size_t)i * prompt_stride;
+      T = std::min(T, std::min(host_n_prompt[i], limit(i) - 1));
+      for (int j = 1; j < T; j++)
+        if (pt[j] == 199999 || pt[j] == 200002) T = j;
+    }
+    if (T >= 2) {
+      std::vector<int> toks((size_t)B * T);
+      for (int i = 0; i < B; i++)
+        memcpy(&toks[(size_t)i * T], host_prompts + (size_t)i * prompt_stride, sizeof(int) * T);
+      int rc = gptoss_engine_prefill(e, toks.data(), B, T, next.data());
+      if (rc != GPTOSS_OK) return rc;
+      for (int i = 0; i < B; i++) cur_pos[i] = T - 1;  // the bookkeeping below finishes position T-1
+      skip_step = 1;
+    }
+  }
+  while (active_count > 0) {
+    if (!skip_step) {
+      int rc = gptoss_engine_step_ragged(e, cur_tok.data(), cur_pos.data(), B, next.data());
+      if (rc != GPTOSS_OK) return rc;
+    }
+    skip_step = 0;
+    for (int i = 0; i < B; i++) {
+      const int r = req[i];
+      if (r < 0) continue;
+      const int *pt = host_prompts + (size_t)r * prompt_stride;
+      const int np = host_n_prompt[r];
+      int *o = host_out + (size_t)r * (max_seq_len + 1);
+      int nt = next[i];
+      if (cur_pos[i] < np - 1) nt = pt[cur_pos[i] + 1];
+      else o[cur_pos[i] - (np - 1)] = nt;
+      cur_tok[i] = nt;
+      cur_pos[i]++;
+      if (nt == 199999 || nt == 200002 || cur_pos[i] >= limit(r) - 1) {
+        finish(i);
+        admit(i);
+      }
+    }
+  }
+  if (n_generated) *n_generated = total;
+  return GPTOSS_OK;
+}
+
+extern "C" int gptoss_engine_generate_ragged(gptoss_engine *e, const int *host_prompts, const int *host_n_prompt,
+                                             int prompt_stride, int n_req, int max_seq_len,
+                                             const int *host_max_len, int *host_out, long long *n_generated) {
+  GPTOSS_REQUIRE(e && host_prompts && host_n_prompt && host_out, GPTOSS_ERR_NULL, "engine_generate: null pointer");
+  GPTOSS_REQUIRE(n_req >= 0 && prompt_stride >= 1 && max_seq_len >= 1 && max_seq_len <= e->max_seq + 1,
+                 GPTOSS_ERR_DIM, "engine_generate: max_seq_len %d needs an engine with max_seq >= %d",
+                 max_seq_len, max_seq_len - 1);
+  for (int r = 0; r < n_req; r++)
+    GPTOSS_REQUIRE(host_n_prompt[r] >= 1 && host_n_prompt[r] <= prompt_stride, GPTOSS_ERR_DIM,
+                   "engine_generate: request %d has %d prompt tokens", r, host_n_prompt[r]);
+  if (host_max_len)
+    for (int r = 0; r < n_req; r++)
+      GPTOSS_REQUIRE(host_max_len[r] >= 1, GPTOSS_ERR_DIM, "engine_generate: request %d has length limit %d", r,
+                     host_max_len[r]);
+  const bool reference_schedule = (e->flags & (GPTOSS_ENGINE_PRECISE | GPTOSS_ENGINE_NO_PREFILL)) != 0;
+  if (reference_schedule) {
+    GPTOSS_REQUIRE(!host_max_len, GPTOSS_ERR_STATE,
+                   "engine_generate: per-request length limits need the continuous schedule "
+                   "(not GPTOSS_ENGINE_PRECISE / GPTOSS_ENGINE_NO_PREFILL)");
+    return generate_lockstep(e, host_prompts, host_n_prompt, prompt_stride, n_req, max_seq_len, host_out, n_generated);
+  }
+  return generate_continuous(e, host_prompts, host_n_prompt, prompt_stride, n_req, max_seq_len, host_max_len,
+                             host_out, n_generated);
+}
+
+extern "C" int gptoss_engine_generate(gptoss_engine *e, const int *host_prompts, const int *host_n_prompt,
+                                      int prompt_stride, int n_req, int max_seq_len, int *host_out,
+                                      long long *n_generated) {
+  return gptoss_engine_generate_ragged(e, host_prompts, host_n_prompt, prompt_stride, n_req, max_seq_len, nullptr,
+                                       host_out, n_generated);
 }
 
 // Device views for tests and tracing: logits of the last step [B,V] and the residual stream.

@@ -63,11 +63,12 @@ __global__ __launch_bounds__(256) void rope_store_kernel(const float *__restrict
                                                          const float *__restrict__ cos_t,
                                                          const float *__restrict__ sin_t, int n_q,
                                                          int n_kv, int D, int cap, int pos0, int T,
-                                                         int store_from) {
-  // row r of the batch is position pos0 + r % T of sequence r / T (T = 1: one lock-step position)
+                                                         int store_from, const int *__restrict__ lens) {
+  // row r of the batch is position pos0 + r % T of sequence r / T (T = 1: one lock-step position),
+  // or, with lens, the last position (lens[r] - 1) of sequence r
   const int r = blockIdx.x;
   const int b = r / T;
-  const int pos = pos0 + (r - b * T);
+  const int pos = lens ? lens[r] - 1 : pos0 + (r - b * T);
   const int half = D >> 1;
   const int q_dim = n_q * D, kv_dim = n_kv * D;
   const float *row = qkv + (size_t)r * (q_dim + 2 * kv_dim);
@@ -221,12 +222,21 @@ int run_rope_store(const float *qkv, float *q_out, bf16_t *kc, bf16_t *vc, const
   return run_rope_store_rows(qkv, q_out, kc, vc, cos_t, sin_t, B, 1, n_q, n_kv, D, cap, pos, 0, s);
 }
 
+int run_rope_store_lens(const float *qkv, float *q_out, bf16_t *kc, bf16_t *vc, const float *cos_t,
+                        const float *sin_t, int B, int n_q, int n_kv, int D, int cap, const int *lens,
+                        hipStream_t s) {
+  TraceScope ts("rope_store", s);
+  rope_store_kernel<<<B, 256, 0, s>>>(qkv, q_out, kc, vc, cos_t, sin_t, n_q, n_kv, D, cap, 0, 1, 0, lens);
+  GPTOSS_LAUNCH_CHECK("rope_store_kernel");
+  return GPTOSS_OK;
+}
+
 int run_rope_store_rows(const float *qkv, float *q_out, bf16_t *kc, bf16_t *vc, const float *cos_t,
                         const float *sin_t, int rows, int T, int n_q, int n_kv, int D, int cap, int pos0,
                         int store_from, hipStream_t s) {
   TraceScope ts("rope_store", s);
   rope_store_kernel<<<rows, 256, 0, s>>>(qkv, q_out, kc, vc, cos_t, sin_t, n_q, n_kv, D, cap, pos0, T,
-                                         store_from);
+                                         store_from, nullptr);
   GPTOSS_LAUNCH_CHECK("rope_store_kernel");
   return GPTOSS_OK;
 }

@@ -16,6 +16,10 @@ int run_rope_store(const float *qkv, float *q_out, bf16_t *kc, bf16_t *vc, const
 int run_rope_store_rows(const float *qkv, float *q_out, bf16_t *kc, bf16_t *vc, const float *cos_t,
                         const float *sin_t, int rows, int T, int n_q, int n_kv, int D, int cap, int pos0,
                         int store_from, hipStream_t s);
+// one row per sequence, each at its own position lens[r] - 1
+int run_rope_store_lens(const float *qkv, float *q_out, bf16_t *kc, bf16_t *vc, const float *cos_t,
+                        const float *sin_t, int B, int n_q, int n_kv, int D, int cap, const int *lens,
+                        hipStream_t s);
 // dst[i, :] = src[i * stride + offset, :]
 int run_gather_rows(const float *src, float *dst, int rows, int n, int stride, int offset, hipStream_t s);
 int run_argmax(const float *logits, int *ids, int B, int V, hipStream_t s);

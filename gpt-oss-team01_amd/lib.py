@@ -78,6 +78,8 @@ SIGNATURES = {
                                   C.POINTER(_vp)]),
     "gptoss_engine_step": (_i, [_vp, _vp, _i, _i, _vp]),
     "gptoss_engine_prefill": (_i, [_vp, _vp, _i, _i, _vp]),
+    "gptoss_engine_step_ragged": (_i, [_vp, _vp, _vp, _i, _vp]),
+    "gptoss_engine_generate_ragged": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp, _vp, C.POINTER(C.c_longlong)]),
     "gptoss_attn_prefill_workspace_bytes": (_sz, [_i, _i, _i, _i, _i, _i]),
     "gptoss_attn_prefill": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _sz, _vp]),
     "gptoss_engine_generate": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp, C.POINTER(C.c_longlong)]),

@@ -283,7 +283,19 @@ class Engine:
                                               nxt.ctypes.data_as(C.c_void_p)))
         return nxt
 
-    def generate(self, prompts, max_seq_len, n_prompt=None):
+    def step_ragged(self, tokens, positions):
+        """One step with every sequence at its own position."""
+        import numpy as np
+        tok = np.ascontiguousarray(tokens, dtype=np.int32)
+        pos = np.ascontiguousarray(positions, dtype=np.int32)
+        nxt = np.empty_like(tok)
+        _l.check(self.L.gptoss_engine_step_ragged(self._h, tok.ctypes.data_as(C.c_void_p),
+                                                  pos.ctypes.data_as(C.c_void_p), tok.size,
+                                                  nxt.ctypes.data_as(C.c_void_p)))
+        return nxt
+
+    def generate(self, prompts, max_seq_len, n_prompt=None, max_len=None):
+        """Greedy generation; max_len (optional, per request) limits a request's total length."""
         import numpy as np
         prompts = np.ascontiguousarray(prompts, dtype=np.int32)
         n_req, stride = prompts.shape
@@ -291,10 +303,17 @@ class Engine:
             np.ascontiguousarray(n_prompt, dtype=np.int32)
         out = np.zeros((n_req, max_seq_len + 1), np.int32)
         n = C.c_longlong(0)
-        _l.check(self.L.gptoss_engine_generate(self._h, prompts.ctypes.data_as(C.c_void_p),
-                                               npr.ctypes.data_as(C.c_void_p), stride, n_req,
-                                               max_seq_len, out.ctypes.data_as(C.c_void_p),
-                                               C.byref(n)))
+        if max_len is None:
+            _l.check(self.L.gptoss_engine_generate(self._h, prompts.ctypes.data_as(C.c_void_p),
+                                                   npr.ctypes.data_as(C.c_void_p), stride, n_req,
+                                                   max_seq_len, out.ctypes.data_as(C.c_void_p),
+                                                   C.byref(n)))
+        else:
+            ml = np.ascontiguousarray(max_len, dtype=np.int32)
+            _l.check(self.L.gptoss_engine_generate_ragged(self._h, prompts.ctypes.data_as(C.c_void_p),
+                                                          npr.ctypes.data_as(C.c_void_p), stride, n_req,
+                                                          max_seq_len, ml.ctypes.data_as(C.c_void_p),
+                                                          out.ctypes.data_as(C.c_void_p), C.byref(n)))
         return out, int(n.value)
 
     def last_logits(self, B):

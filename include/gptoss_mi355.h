@@ -221,9 +221,10 @@ enum {
                                   reference GPU path's bf16 staging: fp32 weights, activations and KV
                                   cache, double-accumulated dot products.  Reproduces the CPU model's
                                   greedy ids; slow, needs host_weights, 4x the weight memory */
-  GPTOSS_ENGINE_NO_PREFILL = 8 /* no prompt-processing buffers: gptoss_engine_generate feeds prompts one
-                                  position per step, as the reference does
-                                  (getp-csrc/submit/getp_run_submit.cpp:60-72) */
+  GPTOSS_ENGINE_NO_PREFILL = 8 /* the reference's schedule, exactly: no prompt-processing buffers,
+                                  gptoss_engine_generate serves requests in batches of max_batch, each
+                                  batch in lock step from position 0, prompts one position per step
+                                  (getp-csrc/submit/getp_run_submit.cpp:13-87) */
 };
 
 /* Build device weights (bf16, packed) and run state for up to max_batch sequences of up to
@@ -238,6 +239,13 @@ int gptoss_engine_create(const gptoss_config *cfg, const float *host_weights, in
  * (getp-csrc/src/model.cpp:6-151).  Synchronises once, to hand the ids back. */
 int gptoss_engine_step(gptoss_engine *e, const int *host_tokens, int pos, int B, int *host_next);
 
+/* The same step with every sequence at its own position host_pos[B] (a scheduler that refills
+ * the slot of a finished sequence while the others carry on).  The reference keeps one scalar pos
+ * for the whole batch (getp-csrc/submit/getp_run_submit.cpp:60); with equal positions this is
+ * gptoss_engine_step.  Not available with GPTOSS_ENGINE_PRECISE. */
+int gptoss_engine_step_ragged(gptoss_engine *e, const int *host_tokens, const int *host_pos, int B,
+                              int *host_next);
+
 /* Positions 0..T-1 of B sequences in one pass: host_tokens int32 [B, T]; fills the KV caches and
  * returns in host_next[B] the arg-max ids after position T-1, i.e. what T calls of
  * gptoss_engine_step with pos = 0..T-1 leave behind (identical ids and caches while no
@@ -251,9 +259,23 @@ int gptoss_engine_prefill(gptoss_engine *e, const int *host_tokens, int B, int T
  * (getp-csrc/submit/getp_run_submit.cpp:60-96): prompts int32 [n_req, prompt_stride] with
  * n_prompt[r] ids each; out int32 [n_req, max_seq_len+1], terminated by -1; returns the harness's
  * generated-token count in *n_generated. */
+/* Unless the engine was created with GPTOSS_ENGINE_PRECISE or GPTOSS_ENGINE_NO_PREFILL the
+ * requests are scheduled continuously: max_batch slots, the prompt positions shared by the first
+ * max_batch requests in one prompt pass, and a slot whose sequence ended (stop id or length limit)
+ * takes the next waiting request at once.  Every request gets the arithmetic it would get alone, so
+ * the output is that of the reference's batch-by-batch lock-step schedule. */
 int gptoss_engine_generate(gptoss_engine *e, const int *host_prompts, const int *host_n_prompt,
                            int prompt_stride, int n_req, int max_seq_len, int *host_out,
                            long long *n_generated);
+
+/* The same with a length limit per request: request r stops after max_len[r] positions in all
+ * (prompt included; capped by max_seq_len), as if it had been run alone with max_seq_len =
+ * max_len[r].  The reference has one limit for all requests (run.cpp `-n`); ragged limits are what
+ * shows the continuous schedule: a batch no longer waits for its longest sequence.  max_len may be
+ * NULL; a non-NULL max_len needs the continuous schedule. */
+int gptoss_engine_generate_ragged(gptoss_engine *e, const int *host_prompts, const int *host_n_prompt,
+                                  int prompt_stride, int n_req, int max_seq_len, const int *max_len,
+                                  int *host_out, long long *n_generated);
 
 void gptoss_engine_destroy(gptoss_engine *e);
 

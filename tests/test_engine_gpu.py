@@ -276,3 +276,60 @@ def test_generate_with_prefill_equals_generate_without(ops, tiny):
     assert np.array_equal(outs[1][0], outs[3][0]) and outs[1][1] == outs[3][1]
     with pytest.raises(Exception):
         ops.Engine(cfg, flat, max_batch=2, max_seq=16, prefill=False).prefill(prompts[:2, :8])
+
+
+def test_step_ragged_equals_lockstep_per_sequence(ops, tiny):
+    """Sequences at different positions in one step: each must get, bit for bit, the logits it gets
+    when the whole batch is at its position (sequence i runs i steps behind sequence 0)."""
+    fx, cfg, flat = tiny
+    prompts = np.asarray(fx["prompts"], np.int32)
+    gold = np.asarray(fx["expected_ids"], np.int32)
+    seqs = np.concatenate([prompts, gold], axis=1)
+    B, n_steps = 6, 30
+    a = ops.Engine(cfg, flat, max_batch=B, max_seq=64)
+    ref = []
+    for pos in range(n_steps):
+        a.step(seqs[:B, pos], pos)
+        ref.append(a.last_logits(B).copy())
+    a.close()
+    b = ops.Engine(cfg, flat, max_batch=B, max_seq=64)
+    lag = np.arange(B)
+    for step in range(n_steps + B - 1):
+        pos = np.clip(step - lag, 0, n_steps - 1)
+        live = (step - lag >= 0) & (step - lag < n_steps)
+        b.step_ragged(seqs[np.arange(B), pos], pos)
+        got = b.last_logits(B)
+        for i in np.nonzero(live)[0]:
+            assert np.array_equal(got[i], ref[pos[i]][i]), (step, i)
+    b.close()
+
+
+def test_continuous_schedule_gives_the_lockstep_output(ops, tiny):
+    """20 requests with ragged prompts and ragged length limits over 4 slots: slots are refilled as
+    their sequences end.  Every request's output must be what it gets when run the reference's way
+    (lock-step batches; a request with a smaller limit produces a prefix), and the token count must
+    be the sum of the per-request counts."""
+    fx, cfg, flat = tiny
+    rng = np.random.default_rng(5)
+    n_req, S = 20, fx["max_seq_len"]
+    prompts = rng.integers(0, cfg.vocab_size, size=(n_req, 24)).astype(np.int32)
+    n_prompt = rng.integers(1, 25, size=n_req).astype(np.int32)
+    max_len = rng.integers(2, S + 1, size=n_req).astype(np.int32)
+    max_len[3] = 1                                              # a request that may not take a step
+    ref = ops.Engine(cfg, flat, max_batch=4, max_seq=S, prefill=False)
+    want, _ = ref.generate(prompts, S, n_prompt=n_prompt)        # everyone runs to the common limit
+    ref.close()
+    eng = ops.Engine(cfg, flat, max_batch=4, max_seq=S)
+    got, n = eng.generate(prompts, S, n_prompt=n_prompt, max_len=max_len)
+    same, n_same = eng.generate(prompts, S, n_prompt=n_prompt)
+    eng.close()
+    assert np.array_equal(same, want)                            # no limits: the lock-step output
+    total = 0
+    for r in range(n_req):
+        gen = max(0, int(max_len[r]) - 1 - int(n_prompt[r]))     # positions left after the prompt
+        total += gen + 1
+        assert got[r, gen + 1] == -1, r
+        assert np.array_equal(got[r, :gen + 1], want[r, :gen + 1]) or gen == 0, r
+        if gen > 0:
+            assert np.array_equal(got[r, :gen], want[r, :gen]), r
+    assert n == total
