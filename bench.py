@@ -29,7 +29,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
 # HBM bytes of one GEMM1 launch at the default workload, from two rocprofv3 --pmc runs of this
 # command (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, the factors the 1 GiB copy below calibrates); the
 # summary is kept in profiles/moe_layer_20b_1024tok_and_decode_attention_kernel_stats_and_hbm_traffic.md
-GEMM1_HBM_TRAFFIC_BYTES = (1_100_961 + 23_041) * 1024
+GEMM1_HBM_TRAFFIC_BYTES = (1_106_309 + 23_041) * 1024
 
 
 def parse():
@@ -43,6 +43,7 @@ def parse():
     ap.add_argument("--no-attn", action="store_true", help="skip the decode-attention figures")
     ap.add_argument("--no-e2e", action="store_true", help="skip the end-to-end decode figure")
     ap.add_argument("--no-mxfp4", action="store_true", help="skip the 120B-shape MXFP4 MoE figure")
+    ap.add_argument("--no-sched", action="store_true", help="skip the scheduler leg of the end-to-end figure")
     return ap.parse_args()
 
 
@@ -283,7 +284,7 @@ def cpu_baseline_attn(ops, torch, n_seq=32):
     return res
 
 
-def bench_e2e(ops, torch, n_req=1024, n_prompt=128, n_decode=256):
+def bench_e2e(ops, torch, n_req=1024, n_prompt=128, n_decode=256, scheduler=True):
     """configs[3]: full GPT-OSS-20B shape, random-init bf16 weights generated on the device,
     1024 prompts of 128 random ids, then 256 greedy decode steps, all sequences in lock step (the
     reference's getp scheduling).  The prompt phase is timed both ways: forced token by token, as
@@ -324,12 +325,13 @@ def bench_e2e(ops, torch, n_req=1024, n_prompt=128, n_decode=256):
     # Scheduler: 4096 requests (32-token prompts, length limits U[64, 384]) over the 1024 slots.
     # Continuous schedule (a finished sequence's slot takes the next request at once) against the
     # reference's batches of 1024 in lock step until the longest sequence of the batch ends.
-    n_sched = 4 * n_req
+    n_sched = 4 * n_req if scheduler else 0
     sp = rng.integers(0, cfg.vocab_size, size=(n_sched, 32), dtype=np.int32)
     limits = rng.integers(64, n_prompt + n_decode + 1, size=n_sched).astype(np.int32)
     useful = int((limits - 1).sum())
     t0 = time.perf_counter()
-    eng.generate(sp, n_prompt + n_decode, max_len=limits)
+    if scheduler:
+        eng.generate(sp, n_prompt + n_decode, max_len=limits)
     t_cont = time.perf_counter() - t0
     t0 = time.perf_counter()
     for b0 in range(0, n_sched, n_req):
@@ -339,7 +341,7 @@ def bench_e2e(ops, torch, n_req=1024, n_prompt=128, n_decode=256):
     t_lock = time.perf_counter() - t0
     sched = {"requests": n_sched, "slots": n_req, "positions": useful,
              "continuous_tok_s": round(useful / t_cont, 1), "lockstep_batches_tok_s": round(useful / t_lock, 1),
-             "workload": "32-token prompts, total length limits U[64,384]"}
+             "workload": "32-token prompts, total length limits U[64,384]"} if scheduler else None
     eng.close()
     return {"decode_tok_s": round(n_req * n_decode / t_decode, 1),
             "decode_ms_per_step": round(t_decode / n_decode * 1e3, 3),
@@ -399,7 +401,7 @@ def main():
                                                        cpu_tokens=min(64, args.cpu_tokens))
     if not args.no_e2e:
         torch.cuda.empty_cache()
-        extra["e2e_20b"] = bench_e2e(ops, torch)
+        extra["e2e_20b"] = bench_e2e(ops, torch, scheduler=not args.no_sched)
 
     if cpu is not None and "e2e_20b" in extra:
         # whole-model CPU figure: not run (84 GB of fp32 weights, minutes per token); scaled from the
