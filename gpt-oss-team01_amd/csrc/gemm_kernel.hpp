@@ -467,9 +467,18 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void grouped_gemm_kernel(GemmParam
   };
   auto decode = [&](int jj) {
     const int work = lo + jj;
-    const int tile = work / p.n_col_tiles;
     Item it;
-    it.ct = work - tile * p.n_col_tiles;
+    int tile;
+    if (p.tiles) {
+      // grouped: column tiles of one row tile are neighbours (the tile's gathered rows stay in L2)
+      tile = work / p.n_col_tiles;
+      it.ct = work - tile * p.n_col_tiles;
+    } else {
+      // dense: row tiles of one column tile are neighbours, so an XCD reads its share of W from
+      // memory once and serves the other row tiles from its L2 (W is the larger operand)
+      it.ct = work / n_tiles;
+      tile = work - it.ct * n_tiles;
+    }
     if (p.tiles) {
       it.mat = p.tiles[1 + 3 * tile];
       it.row0 = p.tiles[2 + 3 * tile];
