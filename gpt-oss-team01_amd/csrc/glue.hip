@@ -54,6 +54,55 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(float *__restrict__ x,
   }
 }
 
+// The same for rows of at most 256 * 4 * VPT floats: every thread keeps its 4 * VPT elements in
+// registers between the two passes and moves them 16 bytes at a time.
+template <int VPT>
+__global__ __launch_bounds__(256) void rmsnorm_rows_kernel(float *__restrict__ x,
+                                                           const float *__restrict__ residual,
+                                                           const float *__restrict__ weight,
+                                                           bf16_t *__restrict__ t_bf16,
+                                                           float *__restrict__ t_f32, int H) {
+  __shared__ double red[4];
+  const size_t row = (size_t)blockIdx.x * H;
+  f32x4 v[VPT];
+  double ss = 0.0;
+#pragma unroll
+  for (int i = 0; i < VPT; i++) {
+    const int h = (threadIdx.x + 256 * i) * 4;
+    v[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (h < H) {
+      v[i] = *reinterpret_cast<const f32x4 *>(x + row + h);
+      if (residual) {
+        const f32x4 r = *reinterpret_cast<const f32x4 *>(residual + row + h);
+#pragma unroll
+        for (int q = 0; q < 4; q++) v[i][q] = __fadd_rn(v[i][q], r[q]);
+        *reinterpret_cast<f32x4 *>(x + row + h) = v[i];
+      }
+#pragma unroll
+      for (int q = 0; q < 4; q++) ss += (double)__fmul_rn(v[i][q], v[i][q]);
+    }
+  }
+  for (int m = 32; m >= 1; m >>= 1) ss += __shfl_xor(ss, m, 64);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
+  __syncthreads();
+  ss = red[0] + red[1] + red[2] + red[3];
+  ss /= H;
+  ss += 1e-5f;
+  const double inv = (double)(1.0f / sqrtf((float)ss));
+#pragma unroll
+  for (int i = 0; i < VPT; i++) {
+    const int h = (threadIdx.x + 256 * i) * 4;
+    if (h < H) {
+      const f32x4 w = *reinterpret_cast<const f32x4 *>(weight + h);
+      f32x4 o;
+#pragma unroll
+      for (int q = 0; q < 4; q++) o[q] = (float)((double)w[q] * (inv * (double)v[i][q]));
+      *reinterpret_cast<u32x2 *>(t_bf16 + row + h) = u32x2{pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3])};
+      if (t_f32) *reinterpret_cast<f32x4 *>(t_f32 + row + h) = o;
+    }
+  }
+}
+
 // Split the fused qkv row, rotate q and k (half-split pairs i, i+D/2; run.cpp:480-499), write q
 // (fp32) and store k, v as bf16 into this layer's cache slot pos % cap.
 // reference: qkv_split_rope_store_kernel, layer_hip_batch.cpp:686-776
@@ -74,23 +123,34 @@ __global__ __launch_bounds__(256) void rope_store_kernel(const float *__restrict
   const float *row = qkv + (size_t)r * (q_dim + 2 * kv_dim);
   const float *cs = cos_t + (size_t)pos * half, *sn = sin_t + (size_t)pos * half;
   const int slot = pos % cap;
+  // four rotation pairs per thread and step: 16-byte loads and stores (half % 4 == 0 for D in {32, 64})
+  const int quads = half >> 2;
+  auto rotate = [&](const float *x, int j4, f32x4 &lo, f32x4 &hi) {
+    const f32x4 x1 = *reinterpret_cast<const f32x4 *>(x + j4), x2 = *reinterpret_cast<const f32x4 *>(x + half + j4);
+    const f32x4 c = *reinterpret_cast<const f32x4 *>(cs + j4), s = *reinterpret_cast<const f32x4 *>(sn + j4);
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+      lo[q] = __fsub_rn(__fmul_rn(x1[q], c[q]), __fmul_rn(x2[q], s[q]));
+      hi[q] = __fadd_rn(__fmul_rn(x2[q], c[q]), __fmul_rn(x1[q], s[q]));
+    }
+  };
   if (q_out != nullptr) {
-    for (int p = threadIdx.x; p < n_q * half; p += 256) {
-      int h = p / half, j = p - h * half;
-      float x1 = row[h * D + j], x2 = row[h * D + half + j];
-      float c = cs[j], s = sn[j];
-      q_out[(size_t)r * q_dim + h * D + j] = __fsub_rn(__fmul_rn(x1, c), __fmul_rn(x2, s));
-      q_out[(size_t)r * q_dim + h * D + half + j] = __fadd_rn(__fmul_rn(x2, c), __fmul_rn(x1, s));
+    for (int p = threadIdx.x; p < n_q * quads; p += 256) {
+      const int h = p / quads, j4 = (p - h * quads) * 4;
+      f32x4 lo, hi;
+      rotate(row + h * D, j4, lo, hi);
+      *reinterpret_cast<f32x4 *>(q_out + (size_t)r * q_dim + h * D + j4) = lo;
+      *reinterpret_cast<f32x4 *>(q_out + (size_t)r * q_dim + h * D + half + j4) = hi;
     }
   }
   if (pos < store_from) return;  // a ring cache keeps only the last positions of a prefill
-  for (int p = threadIdx.x; p < n_kv * half; p += 256) {
-    int g = p / half, j = p - g * half;
-    float x1 = row[q_dim + g * D + j], x2 = row[q_dim + g * D + half + j];
-    float c = cs[j], s = sn[j];
-    size_t base = ((size_t)(b * n_kv + g) * cap + slot) * D;
-    kc[base + j] = f32_to_bf16(__fsub_rn(__fmul_rn(x1, c), __fmul_rn(x2, s)));
-    kc[base + half + j] = f32_to_bf16(__fadd_rn(__fmul_rn(x2, c), __fmul_rn(x1, s)));
+  for (int p = threadIdx.x; p < n_kv * quads; p += 256) {
+    const int g = p / quads, j4 = (p - g * quads) * 4;
+    f32x4 lo, hi;
+    rotate(row + q_dim + g * D, j4, lo, hi);
+    const size_t base = ((size_t)(b * n_kv + g) * cap + slot) * D;
+    *reinterpret_cast<u32x2 *>(kc + base + j4) = u32x2{pack_bf16x2(lo[0], lo[1]), pack_bf16x2(lo[2], lo[3])};
+    *reinterpret_cast<u32x2 *>(kc + base + half + j4) = u32x2{pack_bf16x2(hi[0], hi[1]), pack_bf16x2(hi[2], hi[3])};
   }
   for (int p = threadIdx.x; p < kv_dim; p += 256) {
     int g = p / D, d = p - g * D;
@@ -195,7 +255,13 @@ int run_embedding(const bf16_t *table, const int *tokens, float *x, int B, int H
 int run_rmsnorm(float *x, const float *residual, const float *weight, bf16_t *t_bf16, float *t_f32,
                 int B, int H, hipStream_t s) {
   TraceScope ts(residual ? "residual_rmsnorm" : "rmsnorm", s);
-  rmsnorm_kernel<<<B, 256, 0, s>>>(x, residual, weight, t_bf16, t_f32, H);
+  const bool vec = H % 4 == 0 && aligned(x, 16) && aligned(weight, 16) && aligned(t_bf16, 8) &&
+                   (!residual || aligned(residual, 16)) && (!t_f32 || aligned(t_f32, 16));
+  if (vec && H <= 1024) rmsnorm_rows_kernel<1><<<B, 256, 0, s>>>(x, residual, weight, t_bf16, t_f32, H);
+  else if (vec && H <= 2048) rmsnorm_rows_kernel<2><<<B, 256, 0, s>>>(x, residual, weight, t_bf16, t_f32, H);
+  else if (vec && H <= 3072) rmsnorm_rows_kernel<3><<<B, 256, 0, s>>>(x, residual, weight, t_bf16, t_f32, H);
+  else if (vec && H <= 4096) rmsnorm_rows_kernel<4><<<B, 256, 0, s>>>(x, residual, weight, t_bf16, t_f32, H);
+  else rmsnorm_kernel<<<B, 256, 0, s>>>(x, residual, weight, t_bf16, t_f32, H);
   GPTOSS_LAUNCH_CHECK("rmsnorm_kernel");
   return GPTOSS_OK;
 }
