@@ -216,6 +216,8 @@ __global__ __launch_bounds__(SORT_THREADS) void group_sort_kernel(
   int *hist = smem;                    // [SORT_WAVES][E] per-wave counts, then per-wave cursors
   int *total = hist + SORT_WAVES * E;  // [E]
   int *offs = total + E;               // [E+1]
+  int *cost_pre = offs + E + 1;        // [E] exclusive prefix of the experts' estimated cost
+  int *tile_pre = cost_pre + E;        // [E] first tile of every expert
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const uint64_t lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
 
@@ -301,44 +303,48 @@ __global__ __launch_bounds__(SORT_THREADS) void group_sort_kernel(
     // fall inside a tile (between two of its column tiles), hence the 16-bit fraction.
     if (xcd_bounds != nullptr && tiles != nullptr && rows_per_tile > 0) {
       const int cfull = cost0 + 2 * (rows_per_tile / 32);
-      int cost[4], clast[4], cpre[4];
+      auto last_cost = [&](int count, int n) { return cost0 + 2 * ((count - (n - 1) * rows_per_tile + 31) / 32); };
+      int cost[4], cpre[4];
+#pragma unroll
+      for (int i = 0; i < 4; i++) cost[i] = (nt[i] > 0) ? (nt[i] - 1) * cfull + last_cost(cnt[i], nt[i]) : 0;
+      const int ctot = wave_scan4(cost, cpre);
 #pragma unroll
       for (int i = 0; i < 4; i++) {
-        const int last_rows = cnt[i] - (nt[i] - 1) * rows_per_tile;
-        clast[i] = cost0 + 2 * ((last_rows + 31) / 32);
-        cost[i] = (nt[i] > 0) ? (nt[i] - 1) * cfull + clast[i] : 0;
-      }
-      const int ctot = wave_scan4(cost, cpre);
-      const float rcp_cfull = __builtin_amdgcn_rcpf((float)cfull);
-      // all quantities fit 32 bits: ctot < 2^15 tiles * (cost0 + 16)
-      for (int x = 0; x < 8; x++) {
-        const int target = (x * ctot) >> 3;
-        int pre = -1, nte = 0, cl = 0, te = 0;  // the (at most one) expert of this lane that holds the cut
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-          const bool hit = cost[i] > 0 && cpre[i] <= target && target < cpre[i] + cost[i];
-          pre = hit ? cpre[i] : pre;
-          nte = hit ? nt[i] : nte;
-          cl = hit ? clast[i] : cl;
-          te = hit ? tile_ex[i] : te;
+        const int e = lane * 4 + i;
+        if (e < E) {
+          cost_pre[e] = cpre[i];
+          tile_pre[e] = tile_ex[i];
         }
-        if (pre >= 0) {
+      }
+      // lane x finds cut x: the last expert whose cost prefix is <= x/8 of the total has a tile under
+      // the cut (experts without rows share their successor's prefix).  All quantities fit 32 bits:
+      // ctot < 2^15 tiles * (cost0 + 16).
+      if (lane < 8) {
+        int bound = 0;
+        if (ctot > 0) {
+          const int target = (lane * ctot) >> 3;
+          int lo = 0, hi = E - 1;
+          while (lo < hi) {
+            const int mid = (lo + hi + 1) >> 1;
+            if (cost_pre[mid] <= target) lo = mid;
+            else hi = mid - 1;
+          }
+          const int count = offs[lo + 1] - offs[lo];
+          const int nte = (count + rows_per_tile - 1) / rows_per_tile;
           // float quotient (operands < 2^24) with a one-step correction instead of integer division
-          const int a = target - pre;
+          const int a = target - cost_pre[lo];
+          const float rcp_cfull = __builtin_amdgcn_rcpf((float)cfull);
           int t = (int)((float)a * rcp_cfull);
           t -= (t * cfull > a) ? 1 : 0;
           t += ((t + 1) * cfull <= a) ? 1 : 0;
           t = min(t, nte - 1);
           const int rest = a - t * cfull;
-          const float inv = (t == nte - 1) ? __builtin_amdgcn_rcpf((float)cl) : rcp_cfull;
-          xcd_bounds[x] = ((te + t) << 16) | min(65535, (int)((float)rest * 65536.0f * inv));
+          const float inv = (t == nte - 1) ? __builtin_amdgcn_rcpf((float)last_cost(count, nte)) : rcp_cfull;
+          bound = ((tile_pre[lo] + t) << 16) | min(65535, (int)((float)rest * 65536.0f * inv));
         }
+        xcd_bounds[lane] = bound;
       }
-      if (lane == 0) {
-        xcd_bounds[8] = n_tiles << 16;
-        if (ctot == 0)
-          for (int x = 0; x < 8; x++) xcd_bounds[x] = 0;
-      }
+      if (lane == 0) xcd_bounds[8] = n_tiles << 16;
     }
   }
   __syncthreads();
@@ -456,7 +462,7 @@ static int moe_route_impl(const float *logits, int B, int E, int k, float *topk_
   }
   int nbits = 0;
   while ((1 << nbits) < E) nbits++;
-  size_t smem = sizeof(int) * ((size_t)SORT_WAVES * E + E + (E + 1));
+  size_t smem = sizeof(int) * ((size_t)SORT_WAVES * E + E + (E + 1) + 2 * (size_t)E);
   {
     TraceScope ts("group_sort", s);
     group_sort_kernel<<<1, SORT_THREADS, smem, s>>>(topk_i, B * k, E, nbits, expert_offsets,
