@@ -14,6 +14,10 @@
 //     contiguous per load; position p lives in slot p % capacity (ring buffer for window layers);
 //   * long contexts are cut into chunks (flash-decoding): partial (max, sum, O) per chunk, merged
 //     with the sink by a small second kernel; sequences that fit one chunk finish in the first.
+//     The chunk length depends only on the row's own slot range, so a row's result is the same
+//     whatever else is in the launch;
+//   * several query rows may share one sequence's cache (rows_per_seq), each with its own length:
+//     the T positions of a prompt are T such rows, which is all the prompt-pass attention is.
 #include <algorithm>
 #include <type_traits>
 

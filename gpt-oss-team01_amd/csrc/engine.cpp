@@ -1,6 +1,9 @@
-// Single-GPU decode engine: device weights in kernel layout, run state, one lock-step decode step
-// (the op order of the reference's forward_gpu_20b_batched, getp-csrc/src/model.cpp:6-151) and the
-// greedy generation loop of its getp scheduler (getp-csrc/submit/getp_run_submit.cpp:60-96).
+// Single-GPU decode engine: device weights in kernel layout, run state, one decode step (the op
+// order of the reference's forward_gpu_20b_batched, getp-csrc/src/model.cpp:6-151; all sequences
+// at one position, or each at its own), a prompt pass that runs many positions of a sequence
+// through the same kernels at once, and greedy generation: the reference's lock-step batches
+// (getp-csrc/submit/getp_run_submit.cpp:13-96) or, by default, the same requests over a fixed set
+// of slots that are refilled as sequences end.
 #include <math.h>
 #include <string.h>
 
