@@ -39,6 +39,10 @@ def build(ref: bool = True) -> None:
     subprocess.run(["make", "-s", "-B", "libgptoss_oracle.so"], cwd=HERE, check=True)
     if ref and os.path.exists("/root/reference/run.cpp"):
         subprocess.run(["make", "-s", "-B", "ref"], cwd=HERE, check=True)
+        # the reference's run executable around this repository's getp hooks (needs the product library)
+        pkg = os.path.join(os.path.dirname(HERE), "gpt-oss-team01_amd", "libgptoss_mi355.so")
+        if os.path.exists(pkg):
+            subprocess.run(["make", "-s", "-B", "getp"], cwd=HERE, check=True)
 
 
 _lib = None
