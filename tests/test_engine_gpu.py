@@ -333,3 +333,40 @@ def test_continuous_schedule_gives_the_lockstep_output(ops, tiny):
         if gen > 0:
             assert np.array_equal(got[r, :gen], want[r, :gen]), r
     assert n == total
+
+
+def test_stop_ids_in_prompts_and_schedules_agree(ops, orc, binfmt, synth):
+    """A model with the real vocabulary size (so that the stop ids 199999 and 200002 exist) and
+    prompts that contain them: a forced stop id ends its sequence in the reference's loop
+    (getp_run_submit.cpp:75-83, run.cpp:939-941).  The continuous schedule with the prompt pass,
+    the lock-step schedule and the fp32-faithful engine must all end every sequence where the CPU
+    oracle ends it and report its token count; the two bf16 schedules must agree id for id, and the
+    fp32-faithful engine must reproduce the oracle's ids."""
+    cfg = binfmt.Config(vocab_size=200064, hidden_dim=64, n_experts=4, experts_per_token=2,
+                        intermediate_dim=64, n_layers=2, head_dim=32, n_attn_heads=2, n_kv_heads=1,
+                        seq_len=2048, initial_context_length=4096, rope_theta=150000.0,
+                        rope_scaling_factor=32.0, sliding_window=128, swiglu_limit=7.0)
+    tensors = synth.random_tensors(cfg, 3)
+    flat = np.concatenate([np.asarray(t, np.float32).ravel() for t in tensors.values()])
+    rng = np.random.default_rng(4)
+    n_req, stride, S = 7, 12, 24
+    prompts = rng.integers(0, 199000, size=(n_req, stride)).astype(np.int32)
+    prompts[1, 5] = 199999          # ends in the middle of its prompt
+    prompts[2, 1] = 200002          # ends at the first forced token
+    prompts[3, stride - 1] = 199999  # ends at the last prompt token
+    prompts[5, 0] = 200002          # the first token is never checked
+    prompts[6, 3] = 200002
+    prompts[6, 7] = 199999
+    want, n_want = orc.generate(cfg, flat, prompts, S)
+    ends = (want < 0).argmax(axis=1)
+    outs = {}
+    for name, kw in (("continuous", {}), ("lockstep", {"prefill": False}), ("precise", {"precise": True})):
+        eng = ops.Engine(cfg, flat, max_batch=3, max_seq=S, **kw)      # 7 requests over 3 slots
+        outs[name] = eng.generate(prompts, S)
+        eng.close()
+        got, n = outs[name]
+        assert n == n_want, name
+        assert np.array_equal((got < 0).argmax(axis=1), ends), name
+    assert np.array_equal(outs["continuous"][0], outs["lockstep"][0])
+    assert np.array_equal(outs["precise"][0], want)
+    assert sorted(set(ends.tolist())) != [S - stride + 1]              # some sequences did end early
