@@ -343,6 +343,29 @@ def bench_e2e(ops, torch, n_req=1024, n_prompt=128, n_decode=256, scheduler=True
              "continuous_tok_s": round(useful / t_cont, 1), "lockstep_batches_tok_s": round(useful / t_lock, 1),
              "workload": "32-token prompts, total length limits U[64,384]"} if scheduler else None
     eng.close()
+    # The same model with the experts kept in MXFP4, as GPT-OSS checkpoints hold them (random codes
+    # and scales here): same kernels' bf16 operands, a quarter of the expert bytes per step.
+    eng = ops.Engine(cfg, None, max_batch=n_req, max_seq=n_prompt + n_decode, synthetic=True, seed=1,
+                     keep_logits=False, mxfp4_experts=True)
+    dev_gb_q = eng.device_bytes() / 1e9
+    eng.prefill(prompts[:64])
+    t0 = time.perf_counter()
+    tok = eng.prefill(prompts)
+    t_prefill_q = time.perf_counter() - t0
+    t0 = time.perf_counter()
+    for pos in range(n_prompt, n_prompt + n_decode):
+        tok = eng.step(tok, pos)
+    t_decode_q = time.perf_counter() - t0
+    trace = ops.KernelTrace(capacity=2048)
+    with trace:
+        eng.step(tok, n_prompt + n_decode - 1)
+    qkern = trace.summary()
+    eng.close()
+    mxfp4 = {"decode_tok_s": round(n_req * n_decode / t_decode_q, 1),
+             "decode_ms_per_step": round(t_decode_q / n_decode * 1e3, 3),
+             "prompt_tok_s_prefill": round(n_req * n_prompt / t_prefill_q, 1), "device_gb": round(dev_gb_q, 1),
+             "last_step_kernels_us": {k: [c, round(ms * c * 1e3, 1)] for k, (c, ms) in qkern.items()},
+             "weights": "experts MXFP4 (codes uniform, scale exponents U{-13..-5}), everything else as above"}
     return {"decode_tok_s": round(n_req * n_decode / t_decode, 1),
             "decode_ms_per_step": round(t_decode / n_decode * 1e3, 3),
             "prompt_tok_s_lockstep": round(n_req * (n_prompt - 1) / t_prompt, 1),
@@ -353,6 +376,7 @@ def bench_e2e(ops, torch, n_req=1024, n_prompt=128, n_decode=256, scheduler=True
             "last_step_kernels_us": {k: [c, round(ms * c * 1e3, 1)] for k, (c, ms) in kern.items()},
             "prefill_pass_8192_rows_kernels_us": {k: [c, round(ms * c * 1e3, 1)] for k, (c, ms) in pkern.items()},
             "scheduler": sched,
+            "mxfp4_experts": mxfp4,
             "config": "24 blocks, hidden 2880, 64q/8kv heads x 64, 32 experts top-4, vocab 201088, "
                       "window 128 on even layers; 1024 seqs x (128 prompt + 256 decoded)"}
 

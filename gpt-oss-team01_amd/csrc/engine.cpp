@@ -30,9 +30,9 @@ struct LayerWeights {
   float *sinks;                   // [nq]
   bf16_t *w_router;               // [E,H] row-major
   float *b_router;
-  bf16_t *w1;                     // packed GLU [E][2I,H]
+  bf16_t *w1;                     // packed GLU [E][2I,H] (bf16, or MXFP4 bytes with GPTOSS_ENGINE_MXFP4_EXPERTS)
   float *b1;
-  bf16_t *w2;                     // packed [E][H,I]
+  bf16_t *w2;                     // packed [E][H,I]     (likewise)
   float *b2;
   bf16_t *k_cache, *v_cache;
   int cache_cap;
@@ -95,6 +95,10 @@ struct Builder {
   float *stage_f32 = nullptr;
   bf16_t *stage_bf16 = nullptr;
   size_t stage_elems = 0;
+  // MXFP4 expert storage: unpacked codes and scales of one staging chunk, and the flag the
+  // requantisation kernel raises when a value has no exact MXFP4 representation
+  unsigned char *q_blocks = nullptr, *q_scales = nullptr;
+  int *q_not_exact = nullptr;
 
   template <typename T>
   T *alloc(size_t n) {
@@ -162,6 +166,35 @@ struct Builder {
       hip(hipStreamSynchronize(e->stream), "sync");
     }
     return dst;
+  }
+
+  // fp32 host matrices (exactly MXFP4-representable) or random MXFP4 weights -> packed MXFP4
+  bf16_t *upload_matrices_mxfp4(const float *host, int n_mat, int n_out, int n_in, int pack_flags,
+                                uint64_t seed) {
+    const size_t per = (size_t)n_out * n_in;
+    const size_t mat_bytes = per / 2 + per / 32;
+    unsigned char *dst = alloc<unsigned char>(mat_bytes * n_mat);
+    if (!ok()) return nullptr;
+    if (per > stage_elems) {
+      rc = fail(GPTOSS_ERR_DIM, "engine: a %d x %d matrix exceeds the staging buffer", n_out, n_in);
+      return nullptr;
+    }
+    const int group = (int)std::max<size_t>(1, stage_elems / per);
+    for (int m0 = 0; m0 < n_mat && ok(); m0 += group) {
+      const int nm = std::min(group, n_mat - m0);
+      const size_t n_blocks = per * nm / 32;
+      if (host) {
+        hip(hipMemcpyAsync(stage_f32, host + per * m0, per * nm * sizeof(float), hipMemcpyHostToDevice, e->stream), "H2D");
+        check(run_requant_mxfp4(stage_f32, n_blocks, q_blocks, q_scales, q_not_exact, e->stream));
+      } else {
+        // scale exponents -13..-5: weights of the order of 0.02, as the bf16 synthetic weights
+        check(run_synth_mxfp4(q_blocks, q_scales, n_blocks, seed + 7919ull * (uint64_t)m0, -5, e->stream));
+      }
+      if (!ok()) break;
+      check(gptoss_pack_mxfp4(q_blocks, q_scales, dst + mat_bytes * m0, nm, n_out, n_in, pack_flags, e->stream));
+      hip(hipStreamSynchronize(e->stream), "sync");
+    }
+    return reinterpret_cast<bf16_t *>(dst);
   }
 };
 
@@ -366,6 +399,8 @@ extern "C" int gptoss_engine_create(const gptoss_config *cfg, const float *host_
   const bool synthetic = (flags & GPTOSS_ENGINE_SYNTHETIC) != 0;
   GPTOSS_REQUIRE(synthetic || host_weights, GPTOSS_ERR_NULL, "engine_create: host_weights is NULL");
   const bool precise = (flags & GPTOSS_ENGINE_PRECISE) != 0;
+  GPTOSS_REQUIRE(!(precise && (flags & GPTOSS_ENGINE_MXFP4_EXPERTS)), GPTOSS_ERR_STATE,
+                 "engine_create: GPTOSS_ENGINE_PRECISE keeps fp32 weights (not GPTOSS_ENGINE_MXFP4_EXPERTS)");
   GPTOSS_REQUIRE(!(precise && synthetic), GPTOSS_ERR_STATE,
                  "engine_create: GPTOSS_ENGINE_PRECISE needs host weights (not GPTOSS_ENGINE_SYNTHETIC)");
   const gptoss_config &c = *cfg;
@@ -416,6 +451,13 @@ extern "C" int gptoss_engine_create(const gptoss_config *cfg, const float *host_
   b.stage_elems = std::max<size_t>(biggest, (size_t)16 << 20);
   if (!synthetic) b.hip(hipMalloc((void **)&b.stage_f32, b.stage_elems * sizeof(float)), "staging hipMalloc");
   else b.hip(hipMalloc((void **)&b.stage_bf16, b.stage_elems * sizeof(bf16_t)), "staging hipMalloc");
+  const bool mxfp4 = (flags & GPTOSS_ENGINE_MXFP4_EXPERTS) != 0;
+  if (mxfp4) {
+    b.hip(hipMalloc((void **)&b.q_blocks, b.stage_elems / 2), "staging hipMalloc");
+    b.hip(hipMalloc((void **)&b.q_scales, b.stage_elems / 32), "staging hipMalloc");
+    b.hip(hipMalloc((void **)&b.q_not_exact, sizeof(int)), "staging hipMalloc");
+    if (b.ok()) b.hip(hipMemsetAsync(b.q_not_exact, 0, sizeof(int), e->stream), "memset");
+  }
 
   // walk the .bin payload in file order (reference run.cpp:194-233)
   const float *p = host_weights;
@@ -488,9 +530,11 @@ extern "C" int gptoss_engine_create(const gptoss_config *cfg, const float *host_
     w.sinks = b.upload_f32(at(sinks, nq, l), nq, next_seed(), 0.f, STD);
     w.w_router = b.upload_matrices(at(w_router, (size_t)E * H, l), 1, E, H, false, 0, next_seed(), STD);
     w.b_router = b.upload_f32(at(b_router, E, l), E, next_seed(), 0.f, STD);
-    w.w1 = b.upload_matrices(at(w1, (size_t)E * 2 * I * H, l), E, 2 * I, H, true, GPTOSS_PACK_GLU, next_seed(), STD);
+    w.w1 = mxfp4 ? b.upload_matrices_mxfp4(at(w1, (size_t)E * 2 * I * H, l), E, 2 * I, H, GPTOSS_PACK_GLU, next_seed())
+                 : b.upload_matrices(at(w1, (size_t)E * 2 * I * H, l), E, 2 * I, H, true, GPTOSS_PACK_GLU, next_seed(), STD);
     w.b1 = b.upload_f32(at(b1, (size_t)E * 2 * I, l), (size_t)E * 2 * I, next_seed(), 0.f, STD);
-    w.w2 = b.upload_matrices(at(w2, (size_t)E * H * I, l), E, H, I, true, 0, next_seed(), STD);
+    w.w2 = mxfp4 ? b.upload_matrices_mxfp4(at(w2, (size_t)E * H * I, l), E, H, I, 0, next_seed())
+                 : b.upload_matrices(at(w2, (size_t)E * H * I, l), E, H, I, true, 0, next_seed(), STD);
     w.b2 = b.upload_f32(at(b2, (size_t)E * H, l), (size_t)E * H, next_seed(), 0.f, STD);
     // even layers keep only the sliding window (ring buffer), odd layers the whole context
     // (reference run.cpp:582, getp-csrc/src/alloc.cpp:245-250)
@@ -505,8 +549,18 @@ extern "C" int gptoss_engine_create(const gptoss_config *cfg, const float *host_
       b.hip(hipMemsetAsync(w.v_cache, 0, cache_elems * 2, e->stream), "memset");
     }
   }
+  if (mxfp4 && b.ok()) {
+    int not_exact = 0;
+    b.hip(hipMemcpy(&not_exact, b.q_not_exact, sizeof(int), hipMemcpyDeviceToHost), "D2H");
+    if (b.ok() && not_exact)
+      b.rc = fail(GPTOSS_ERR_STATE, "engine_create: GPTOSS_ENGINE_MXFP4_EXPERTS needs expert weights that are exactly "
+                                    "representable in MXFP4 (e2m1 codes, one power-of-two scale per 32 inputs)");
+  }
   if (b.stage_f32) (void)hipFree(b.stage_f32);
   if (b.stage_bf16) (void)hipFree(b.stage_bf16);
+  if (b.q_blocks) (void)hipFree(b.q_blocks);
+  if (b.q_scales) (void)hipFree(b.q_scales);
+  if (b.q_not_exact) (void)hipFree(b.q_not_exact);
 
   // rotary tables
   {
@@ -644,7 +698,10 @@ static int step_impl(gptoss_engine *e, const int *host_tokens, int pos, const in
     mw.w2 = w.w2;
     mw.b2 = w.b2;
     // x += MoE branch (the combine kernel adds into the residual stream, model.cpp:121-131)
-    STEP(gptoss_moe_forward(&mw, e->t, B, e->x, 1, e->moe_ws, e->moe_ws_bytes, s));
+    if (e->flags & GPTOSS_ENGINE_MXFP4_EXPERTS)
+      STEP(gptoss_moe_forward_mxfp4(&mw, e->t, B, e->x, 1, e->moe_ws, e->moe_ws_bytes, s));
+    else
+      STEP(gptoss_moe_forward(&mw, e->t, B, e->x, 1, e->moe_ws, e->moe_ws_bytes, s));
     // next layer's attention norm, or the final norm
     const float *nw = (l + 1 < L) ? e->layers[l + 1].attn_norm : e->final_norm;
     STEP(run_rmsnorm(e->x, nullptr, nw, e->t, nullptr, B, H, s));
@@ -743,7 +800,10 @@ static int prefill_chunk(gptoss_engine *e, const int *host_tokens, int seq0, int
     mw.b1 = w.b1;
     mw.w2 = w.w2;
     mw.b2 = w.b2;
-    STEP(gptoss_moe_forward(&mw, pf.t, rows, pf.x, 1, pf.moe_ws, pf.moe_ws_bytes, s));
+    if (e->flags & GPTOSS_ENGINE_MXFP4_EXPERTS)
+      STEP(gptoss_moe_forward_mxfp4(&mw, pf.t, rows, pf.x, 1, pf.moe_ws, pf.moe_ws_bytes, s));
+    else
+      STEP(gptoss_moe_forward(&mw, pf.t, rows, pf.x, 1, pf.moe_ws, pf.moe_ws_bytes, s));
     if (l + 1 < L) STEP(run_rmsnorm(pf.x, nullptr, e->layers[l + 1].attn_norm, pf.t, nullptr, rows, H, s));
   }
   // only the last position of every sequence goes through the final norm and the classifier

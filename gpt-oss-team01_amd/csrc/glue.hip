@@ -240,6 +240,67 @@ __global__ __launch_bounds__(256) void synth_normal_f32_kernel(float *__restrict
     dst[i] = bf16_to_f32(f32_to_bf16(mean + std * normal_at(seed, i)));
 }
 
+// fp32 -> MXFP4, exact or not at all.  One thread per block of 32 consecutive inputs of a row:
+// the scale is the smallest power of two that brings the block's largest magnitude to at most 6
+// (any block that has an exact e2m1 representation under some scale also has one under this,
+// the finest, scale); every value must then equal sign * {0,.5,1,1.5,2,3,4,6} * scale, otherwise
+// *not_exact is set.  blocks [n_blocks, 16]: byte j = elements 2j (low nibble), 2j+1 (high nibble);
+// scales [n_blocks] e8m0 (the checkpoint layout, export_model_bin/gpt-oss-20b/export_model_bin.py:66-123).
+__global__ __launch_bounds__(256) void requant_mxfp4_kernel(const float *__restrict__ src, size_t n_blocks,
+                                                            unsigned char *__restrict__ blocks,
+                                                            unsigned char *__restrict__ scales,
+                                                            int *__restrict__ not_exact) {
+  for (size_t b = (size_t)blockIdx.x * 256 + threadIdx.x; b < n_blocks; b += (size_t)gridDim.x * 256) {
+    const f32x4 *sp = reinterpret_cast<const f32x4 *>(src + b * 32);
+    float v[32];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      const f32x4 q = sp[i];
+      v[4 * i] = q[0], v[4 * i + 1] = q[1], v[4 * i + 2] = q[2], v[4 * i + 3] = q[3];
+    }
+    float mx = 0.f;
+#pragma unroll
+    for (int i = 0; i < 32; i++) mx = fmaxf(mx, fabsf(v[i]));
+    int e = 0;  // scale = 2^e
+    if (mx > 0.f) {
+      int ex;
+      const float m = frexpf(mx, &ex);  // mx = m * 2^ex, m in [0.5, 1)
+      // mx / 2^e <= 6 = 0.75 * 2^3  <=>  e >= ex - 3 when m <= 0.75, else e >= ex - 2
+      e = (m <= 0.75f) ? ex - 3 : ex - 2;
+    }
+    bool bad = !(mx < INFINITY) || e < -120 || e > 120;
+    const float inv = ldexpf(1.0f, -e);
+    uint32_t packed[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int i = 0; i < 32; i++) {
+      const float a = fabsf(v[i]) * inv;  // exact: a power-of-two factor
+      // codes 0..7 = 0, .5, 1, 1.5, 2, 3, 4, 6
+      int code = (a <= 2.0f) ? (int)(a * 2.0f) : (a <= 4.0f ? (int)a + 2 : 7);
+      const float back = (code <= 4) ? 0.5f * code : (code == 5 ? 3.0f : (code == 6 ? 4.0f : 6.0f));
+      bad = bad || back != a;
+      code |= (__float_as_uint(v[i]) >> 31) << 3;
+      packed[i >> 3] |= (uint32_t)code << (4 * (i & 7));
+    }
+    *reinterpret_cast<u32x4 *>(blocks + b * 16) = u32x4{packed[0], packed[1], packed[2], packed[3]};
+    scales[b] = (unsigned char)(e + 127);
+    if (bad) *not_exact = 1;
+  }
+}
+
+// random MXFP4 weights: codes uniform over the 16 values, scale exponents uniform in [e_hi - 8, e_hi]
+__global__ __launch_bounds__(256) void synth_mxfp4_kernel(unsigned char *__restrict__ blocks,
+                                                          unsigned char *__restrict__ scales,
+                                                          size_t n_blocks, uint64_t seed, int e_hi) {
+  for (size_t b = (size_t)blockIdx.x * 256 + threadIdx.x; b < n_blocks; b += (size_t)gridDim.x * 256) {
+    const uint64_t r0 = splitmix64(seed * 0xD1342543DE82EF95ull + 3 * b);
+    const uint64_t r1 = splitmix64(seed * 0xD1342543DE82EF95ull + 3 * b + 1);
+    const uint64_t r2 = splitmix64(seed * 0xD1342543DE82EF95ull + 3 * b + 2);
+    *reinterpret_cast<u32x4 *>(blocks + b * 16) =
+        u32x4{(uint32_t)r0, (uint32_t)(r0 >> 32), (uint32_t)r1, (uint32_t)(r1 >> 32)};
+    scales[b] = (unsigned char)(127 + e_hi - (int)(r2 % 9));
+  }
+}
+
 static inline int grid_for(size_t n) {
   size_t g = (n + 255) / 256;
   return (int)(g > 65536 ? 65536 : (g == 0 ? 1 : g));
@@ -371,6 +432,20 @@ int run_f32_to_bf16(const float *src, bf16_t *dst, size_t n, hipStream_t s) {
 int run_fill_int(int *dst, int n, int value, hipStream_t s) {
   fill_int_kernel<<<cdiv(n, 256), 256, 0, s>>>(dst, n, value);
   GPTOSS_LAUNCH_CHECK("fill_int_kernel");
+  return GPTOSS_OK;
+}
+
+int run_requant_mxfp4(const float *src, size_t n_blocks, unsigned char *blocks, unsigned char *scales,
+                      int *not_exact, hipStream_t s) {
+  requant_mxfp4_kernel<<<grid_for(n_blocks), 256, 0, s>>>(src, n_blocks, blocks, scales, not_exact);
+  GPTOSS_LAUNCH_CHECK("requant_mxfp4_kernel");
+  return GPTOSS_OK;
+}
+
+int run_synth_mxfp4(unsigned char *blocks, unsigned char *scales, size_t n_blocks, uint64_t seed, int e_hi,
+                    hipStream_t s) {
+  synth_mxfp4_kernel<<<grid_for(n_blocks), 256, 0, s>>>(blocks, scales, n_blocks, seed, e_hi);
+  GPTOSS_LAUNCH_CHECK("synth_mxfp4_kernel");
   return GPTOSS_OK;
 }
 

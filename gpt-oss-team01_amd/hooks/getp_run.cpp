@@ -44,8 +44,11 @@ void warm_up(Transformer *transformer, Tokenizer *tokenizer) {
   // GPTOSS_PRECISE=1: the CPU model's fp32/double arithmetic on the GPU (exact greedy ids, slow)
   const char *precise = getenv("GPTOSS_PRECISE");
   const char *lockstep = getenv("GPTOSS_NO_PREFILL");  // prompts one position per step, as the reference
+  // GPTOSS_MXFP4=1: experts stored in MXFP4 (exact for GPT-OSS checkpoints, a quarter of the bytes)
+  const char *mxfp4 = getenv("GPTOSS_MXFP4");
   const int flags = ((precise && atoi(precise) != 0) ? GPTOSS_ENGINE_PRECISE : 0) |
-                    ((lockstep && atoi(lockstep) != 0) ? GPTOSS_ENGINE_NO_PREFILL : 0);
+                    ((lockstep && atoi(lockstep) != 0) ? GPTOSS_ENGINE_NO_PREFILL : 0) |
+                    ((mxfp4 && atoi(mxfp4) != 0) ? GPTOSS_ENGINE_MXFP4_EXPERTS : 0);
   if (gptoss_engine_create(&cfg, weights, max_batch, g_gptoss_max_seq, flags, 0, &g_gptoss_engine) != GPTOSS_OK)
     gptoss_die("engine_create");
 }

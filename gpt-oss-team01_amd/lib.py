@@ -21,6 +21,7 @@ ENGINE_SYNTHETIC = 1
 ENGINE_PRECISE = 2
 ENGINE_LOGITS = 4
 ENGINE_NO_PREFILL = 8
+ENGINE_MXFP4_EXPERTS = 16
 
 
 class GptossError(RuntimeError):

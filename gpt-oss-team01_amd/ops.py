@@ -247,14 +247,15 @@ class Engine:
     """Single-GPU decode engine over a flat ``.bin`` payload (or synthetic on-device weights)."""
 
     def __init__(self, cfg, weights_flat=None, max_batch=8, max_seq=64, synthetic=False,
-                 precise=False, seed=0, keep_logits=True, prefill=True):
+                 precise=False, seed=0, keep_logits=True, prefill=True, mxfp4_experts=False):
         _need_gpu()
         import numpy as np
         self.L = _l.load()
         self.cfg = cfg
         self.max_batch, self.max_seq = max_batch, max_seq
         flags = (_l.ENGINE_SYNTHETIC if synthetic else 0) | (_l.ENGINE_PRECISE if precise else 0) | \
-            (_l.ENGINE_LOGITS if keep_logits else 0) | (0 if prefill else _l.ENGINE_NO_PREFILL)
+            (_l.ENGINE_LOGITS if keep_logits else 0) | (0 if prefill else _l.ENGINE_NO_PREFILL) | \
+            (_l.ENGINE_MXFP4_EXPERTS if mxfp4_experts else 0)
         self._cc = _l.Config.from_config(cfg)
         wp = None
         if not synthetic:

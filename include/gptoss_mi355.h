@@ -221,10 +221,17 @@ enum {
                                   reference GPU path's bf16 staging: fp32 weights, activations and KV
                                   cache, double-accumulated dot products.  Reproduces the CPU model's
                                   greedy ids; slow, needs host_weights, 4x the weight memory */
-  GPTOSS_ENGINE_NO_PREFILL = 8 /* the reference's schedule, exactly: no prompt-processing buffers,
+  GPTOSS_ENGINE_NO_PREFILL = 8, /* the reference's schedule, exactly: no prompt-processing buffers,
                                   gptoss_engine_generate serves requests in batches of max_batch, each
                                   batch in lock step from position 0, prompts one position per step
                                   (getp-csrc/submit/getp_run_submit.cpp:13-87) */
+  GPTOSS_ENGINE_MXFP4_EXPERTS = 16 /* keep the expert matrices in MXFP4 (0.53 bytes per weight instead of
+                                  2).  GPT-OSS checkpoints are MXFP4 at the source and the .bin holds
+                                  their dequantised values (export_model_bin/gpt-oss-20b/
+                                  export_model_bin.py:66-123), so the fp32 payload converts back
+                                  exactly and the kernels multiply the same bf16 operands: results are
+                                  bit-identical to the bf16 storage.  Creation fails with
+                                  GPTOSS_ERR_STATE if a value has no exact MXFP4 representation. */
 };
 
 /* Build device weights (bf16, packed) and run state for up to max_batch sequences of up to

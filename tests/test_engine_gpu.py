@@ -370,3 +370,41 @@ def test_stop_ids_in_prompts_and_schedules_agree(ops, orc, binfmt, synth):
     assert np.array_equal(outs["continuous"][0], outs["lockstep"][0])
     assert np.array_equal(outs["precise"][0], want)
     assert sorted(set(ends.tolist())) != [S - stride + 1]              # some sequences did end early
+
+
+def test_mxfp4_expert_storage_is_bit_identical_to_bf16_storage(ops, orc, tiny, synth, binfmt):
+    """GPT-OSS expert weights are MXFP4 at the source and the .bin holds their dequantised values.
+    With such a payload GPTOSS_ENGINE_MXFP4_EXPERTS converts the experts back to MXFP4 exactly, and
+    every step must give the logits of the bf16 storage bit for bit (same bf16 operands, same MFMA
+    order), in lock step, through the prompt pass and in generation (the bf16 storage is what the
+    other tests hold against the oracle).  A payload that is not representable must be refused."""
+    fx, cfg, _ = tiny
+    lib = __import__("conftest").load_pkg("lib")
+    rng = np.random.default_rng(21)
+    tensors = synth.random_tensors(cfg, 5)
+    L, E, H, I = cfg.n_layers, cfg.n_experts, cfg.hidden_dim, cfg.intermediate_dim
+    for name, (n_out, n_in) in (("mlp1_weight", (2 * I, H)), ("mlp2_weight", (H, I))):
+        blocks = rng.integers(0, 256, size=(L * E * n_out * n_in // 32, 16), dtype=np.uint8)
+        scales = (127 + rng.integers(-9, -3, size=L * E * n_out * n_in // 32)).astype(np.uint8)
+        blocks[:7] = 0                                     # an all-zero block, zeros next to large codes
+        tensors[name] = orc.mxfp4_dequant(blocks, scales).reshape(L, E, n_out, n_in)
+    flat = np.concatenate([np.asarray(tensors[n], np.float32).ravel() for n in binfmt.tensor_shapes(cfg)])
+    prompts = np.asarray(fx["prompts"], np.int32)
+    B, T = 8, 20
+    a = ops.Engine(cfg, flat, max_batch=B, max_seq=64)
+    b = ops.Engine(cfg, flat, max_batch=B, max_seq=64, mxfp4_experts=True)
+    assert b.device_bytes() < a.device_bytes()
+    for pos in range(T):
+        na, nb = a.step(prompts[:, pos], pos), b.step(prompts[:, pos], pos)
+        assert np.array_equal(na, nb), pos
+        assert np.array_equal(a.last_logits(B), b.last_logits(B)), pos
+    assert np.array_equal(a.prefill(prompts[:, :T]), b.prefill(prompts[:, :T]))
+    assert np.array_equal(a.last_logits(B), b.last_logits(B))
+    ga, gb = a.generate(prompts, fx["max_seq_len"]), b.generate(prompts, fx["max_seq_len"])
+    assert np.array_equal(ga[0], gb[0]) and ga[1] == gb[1]
+    a.close()
+    b.close()
+    # the golden model's experts are bf16-rounded normals: no exact MXFP4 form
+    with pytest.raises(lib.GptossError) as ei:
+        ops.Engine(cfg, tiny[2], max_batch=2, max_seq=16, mxfp4_experts=True)
+    assert ei.value.code == 6 or "MXFP4" in str(ei.value)
