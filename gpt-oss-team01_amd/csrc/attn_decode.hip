@@ -14,8 +14,8 @@
 //     contiguous per load; position p lives in slot p % capacity (ring buffer for window layers);
 //   * long contexts are cut into chunks (flash-decoding): partial (max, sum, O) per chunk, merged
 //     with the sink by a small second kernel; sequences that fit one chunk finish in the first.
-//     The chunk length depends only on the row's own slot range, so a row's result is the same
-//     whatever else is in the launch;
+//     The chunk length is a constant, so a row's result is the same whatever else is in the
+//     launch;
 //   * several query rows may share one sequence's cache (rows_per_seq), each with its own length:
 //     the T positions of a prompt are T such rows, which is all the prompt-pass attention is.
 #include <algorithm>
@@ -48,9 +48,12 @@ struct SeqRange {
   int chunk, nchunks;  // slots per work item, number of work items
 };
 
-// Slots per work item as a function of the row's own slot range, so that a row's result does not
-// depend on what else is in the launch (one lock-step position or many positions of a prefill).
-__host__ __device__ __forceinline__ int attn_chunk_tokens(int span) { return span > 1024 ? 512 : 256; }
+// Slots per work item: a constant, so that a row's result does not depend on what else is in the
+// launch (one lock-step position or many positions of a prefill).  512 keeps contexts of up to
+// 512 positions in one work item (no partial results, no merge kernel), which is what a batch of
+// a thousand sequences wants; a single long sequence still gets one work item per 512 slots and
+// kv head.
+constexpr int ATT_CHUNK = 512;
 
 __device__ __forceinline__ SeqRange seq_range(int len, int cap, int window, int max_len) {
   SeqRange r;
@@ -65,7 +68,7 @@ __device__ __forceinline__ SeqRange seq_range(int len, int cap, int window, int 
     r.s_begin = 0;
     r.s_end = cap;
   }
-  r.chunk = attn_chunk_tokens(r.s_end - r.s_begin);
+  r.chunk = ATT_CHUNK;
   r.nchunks = max(1, (r.s_end - r.s_begin + r.chunk - 1) / r.chunk);
   return r;
 }
@@ -372,11 +375,10 @@ struct AttnPlan {
 
 static AttnPlan attn_plan(int B, int n_q, int D, int max_len) {
   AttnPlan pl;
-  // most work items any row can have: rows choose their chunk length from their own slot range,
-  // which can start up to 63 slots before the first active position
+  // most work items any row can have: a slot range can start up to 63 slots before the first
+  // active position
   const int longest = max_len + ATT_BLOCK - 1;
-  pl.max_chunks = (longest + attn_chunk_tokens(longest) - 1) / attn_chunk_tokens(longest);
-  if (longest > 1024) pl.max_chunks = std::max(pl.max_chunks, (1024 + 255) / 256);
+  pl.max_chunks = (longest + ATT_CHUNK - 1) / ATT_CHUNK;
   if (pl.max_chunks < 1) pl.max_chunks = 1;
   pl.part_o_bytes = align_up((size_t)B * pl.max_chunks * n_q * D * sizeof(float), 256);
   pl.part_ml_bytes = align_up((size_t)B * pl.max_chunks * n_q * 2 * sizeof(float), 256);
@@ -413,7 +415,8 @@ extern "C" int gptoss_kv_cache_write(void *k_cache, void *v_cache, const void *k
 
 extern "C" size_t gptoss_attn_workspace_bytes(int B, int n_q, int n_kv, int head_dim, int max_len) {
   if (B <= 0 || n_q <= 0 || n_kv <= 0 || head_dim <= 0 || max_len <= 0) return 0;
-  // sized for the smallest chunk length so that any window/capacity combination fits
+  // sized for a split into 256-slot work items, twice as fine as the kernel's: any window/capacity
+  // combination fits
   int max_chunks = (max_len + ATT_BLOCK - 1 + 255) / 256;
   return align_up((size_t)B * max_chunks * n_q * head_dim * sizeof(float), 256) +
          align_up((size_t)B * max_chunks * n_q * 2 * sizeof(float), 256);
