@@ -697,14 +697,14 @@ static int step_impl(gptoss_engine *e, const int *host_tokens, int pos, const in
     mw.b1 = w.b1;
     mw.w2 = w.w2;
     mw.b2 = w.b2;
-    // x += MoE branch (the combine kernel adds into the residual stream, model.cpp:121-131)
-    if (e->flags & GPTOSS_ENGINE_MXFP4_EXPERTS)
-      STEP(gptoss_moe_forward_mxfp4(&mw, e->t, B, e->x, 1, e->moe_ws, e->moe_ws_bytes, s));
-    else
-      STEP(gptoss_moe_forward(&mw, e->t, B, e->x, 1, e->moe_ws, e->moe_ws_bytes, s));
-    // next layer's attention norm, or the final norm
+    // x += MoE branch (the combine kernel adds into the residual stream, model.cpp:121-131), and
+    // the next layer's attention norm (or the final norm) of the updated rows in the same kernel
     const float *nw = (l + 1 < L) ? e->layers[l + 1].attn_norm : e->final_norm;
-    STEP(run_rmsnorm(e->x, nullptr, nw, e->t, nullptr, B, H, s));
+    const int q4 = (e->flags & GPTOSS_ENGINE_MXFP4_EXPERTS) ? 1 : 0;
+    const bool fused = combine_norm_applies(H, nw, e->t);
+    STEP(moe_forward_norm(&mw, e->t, B, e->x, e->moe_ws, e->moe_ws_bytes, s, q4, fused ? nw : nullptr,
+                          fused ? e->t : nullptr));
+    if (!fused) STEP(run_rmsnorm(e->x, nullptr, nw, e->t, nullptr, B, H, s));
   }
   if (e->logits) {
     STEP(dense_gemm(e->t, e->unembedding, nullptr, e->logits, EPI_F32, B, V, H, s));
@@ -800,11 +800,12 @@ static int prefill_chunk(gptoss_engine *e, const int *host_tokens, int seq0, int
     mw.b1 = w.b1;
     mw.w2 = w.w2;
     mw.b2 = w.b2;
-    if (e->flags & GPTOSS_ENGINE_MXFP4_EXPERTS)
-      STEP(gptoss_moe_forward_mxfp4(&mw, pf.t, rows, pf.x, 1, pf.moe_ws, pf.moe_ws_bytes, s));
-    else
-      STEP(gptoss_moe_forward(&mw, pf.t, rows, pf.x, 1, pf.moe_ws, pf.moe_ws_bytes, s));
-    if (l + 1 < L) STEP(run_rmsnorm(pf.x, nullptr, e->layers[l + 1].attn_norm, pf.t, nullptr, rows, H, s));
+    const float *nw = (l + 1 < L) ? e->layers[l + 1].attn_norm : nullptr;  // the last rows are normed below
+    const int q4 = (e->flags & GPTOSS_ENGINE_MXFP4_EXPERTS) ? 1 : 0;
+    const bool fused = nw && combine_norm_applies(H, nw, pf.t);
+    STEP(moe_forward_norm(&mw, pf.t, rows, pf.x, pf.moe_ws, pf.moe_ws_bytes, s, q4, fused ? nw : nullptr,
+                          fused ? pf.t : nullptr));
+    if (nw && !fused) STEP(run_rmsnorm(pf.x, nullptr, nw, pf.t, nullptr, rows, H, s));
   }
   // only the last position of every sequence goes through the final norm and the classifier
   STEP(run_gather_rows(pf.x, e->x, Bc, H, T, T - 1, s));

@@ -29,8 +29,18 @@ struct GemmParams {
 // (mat,row-tile) items.
 int run_gemm(const GemmParams &p, bool gather, int epi, int rows_per_tile, int max_tiles,
              hipStream_t s);
+// norm_w / norm_out (optional, accumulate only): also write RMSNorm(out) * norm_w as bf16.  Returns
+// with only the combine done when the fused form does not apply (H > 4096 or misaligned); the
+// caller checks with combine_norm_applies().
 int run_combine(const float *y2, const float *topk_w, const int *inv_perm, float *out, int B, int H,
-                int k, int accumulate, hipStream_t s);
+                int k, int accumulate, const float *norm_w, bf16_t *norm_out, hipStream_t s);
+inline bool combine_norm_applies(int H, const float *norm_w, const bf16_t *norm_out) {
+  return norm_w && norm_out && H % 4 == 0 && H <= 4096 && aligned(norm_w, 16) && aligned(norm_out, 8);
+}
+// The MoE block with the RMSNorm of the updated residual stream fused into its last kernel
+// (moe_layer.cpp); out is accumulated into.
+int moe_forward_norm(const gptoss_moe_weights *w, const void *t, int B, float *out, void *workspace,
+                     size_t workspace_bytes, hipStream_t s, int mxfp4, const float *norm_w, bf16_t *norm_out);
 int moe_rows_per_tile(int B, int k, int E, bool mxfp4);
 int gemm_col_tiles(int N);  // column tiles of one workgroup's width
 // moe_route.hip

@@ -50,6 +50,81 @@ __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ 
   }
 }
 
+// The same combine followed by the RMSNorm of the updated row (the next block's input norm), for
+// rows of at most 1024 * VPT floats: every thread keeps its elements in registers between the two
+// steps.  Element-to-thread mapping, the double-precision sum of squares and the scaling are those
+// of rmsnorm_rows_kernel (glue.hip), so the result equals running the two kernels one after the
+// other bit for bit.
+template <int VPT>
+__global__ __launch_bounds__(256) void combine_norm_kernel(const float *__restrict__ y2,
+                                                           const float *__restrict__ topk_w,
+                                                           const int *__restrict__ inv_perm,
+                                                           float *__restrict__ out, int H, int k,
+                                                           const float *__restrict__ norm_w,
+                                                           bf16_t *__restrict__ t_bf16) {
+  __shared__ double red[4];
+  const int b = blockIdx.x;
+  int rows[8];
+  float w[8];
+#pragma unroll
+  for (int s = 0; s < 8; s++) {
+    rows[s] = (s < k) ? inv_perm[(size_t)b * k + s] : 0x7fffffff;
+    w[s] = (s < k) ? topk_w[(size_t)b * k + s] : 0.f;
+  }
+#pragma unroll
+  for (int i = 0; i < 8; i++)
+#pragma unroll
+    for (int j = 0; j + 1 < 8 - i; j++)
+      if (rows[j] > rows[j + 1]) {
+        int tr = rows[j]; rows[j] = rows[j + 1]; rows[j + 1] = tr;
+        float tw = w[j]; w[j] = w[j + 1]; w[j + 1] = tw;
+      }
+  f32x4 v[VPT];
+  double ss = 0.0;
+#pragma unroll
+  for (int i = 0; i < VPT; i++) {
+    const int h = (threadIdx.x + 256 * i) * 4;
+    v[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (h < H) {
+      f32x4 agg = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s = 0; s < 8; s++) {
+        if (s < k) {
+          const f32x4 y = *reinterpret_cast<const f32x4 *>(y2 + (size_t)rows[s] * H + h);
+#pragma unroll
+          for (int q = 0; q < 4; q++) agg[q] = __fadd_rn(agg[q], __fmul_rn(y[q], w[s]));
+        }
+      }
+      f32x4 *op = reinterpret_cast<f32x4 *>(out + (size_t)b * H + h);
+      const f32x4 prev = *op;
+#pragma unroll
+      for (int q = 0; q < 4; q++) v[i][q] = __fadd_rn(prev[q], agg[q]);
+      *op = v[i];
+#pragma unroll
+      for (int q = 0; q < 4; q++) ss += (double)__fmul_rn(v[i][q], v[i][q]);
+    }
+  }
+  for (int m = 32; m >= 1; m >>= 1) ss += __shfl_xor(ss, m, 64);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
+  __syncthreads();
+  ss = red[0] + red[1] + red[2] + red[3];
+  ss /= H;
+  ss += 1e-5f;
+  const double inv = (double)(1.0f / sqrtf((float)ss));
+#pragma unroll
+  for (int i = 0; i < VPT; i++) {
+    const int h = (threadIdx.x + 256 * i) * 4;
+    if (h < H) {
+      const f32x4 nw = *reinterpret_cast<const f32x4 *>(norm_w + h);
+      f32x4 o;
+#pragma unroll
+      for (int q = 0; q < 4; q++) o[q] = (float)((double)nw[q] * (inv * (double)v[i][q]));
+      *reinterpret_cast<u32x2 *>(t_bf16 + (size_t)b * H + h) =
+          u32x2{pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3])};
+    }
+  }
+}
+
 // Repack row-major [n_out, n_in] matrices into fragment order:
 //   dst[((nb*KS + ks)*64 + lane)*8 + j] = W[row(nb*32 + lane%32)][ks*16 + (lane/32)*8 + j]
 // With GLU pairing, virtual row v of a 32-row block maps to pair (v/32)*16 + v%16, gate for the
@@ -147,8 +222,18 @@ int run_gemm(const GemmParams &p, bool gather, int epi, int rows_per_tile, int m
 }
 
 int run_combine(const float *y2, const float *topk_w, const int *inv_perm, float *out, int B, int H,
-                int k, int accumulate, hipStream_t s) {
+                int k, int accumulate, const float *norm_w, bf16_t *norm_out, hipStream_t s) {
   if (B == 0) return GPTOSS_OK;
+  // out += combine, then norm_out = RMSNorm(out) * norm_w in the same kernel, when asked for
+  if (norm_w && norm_out && accumulate && H % 4 == 0 && H <= 4096 && aligned(norm_w, 16) && aligned(norm_out, 8)) {
+    TraceScope ts("combine_rmsnorm", s);
+    if (H <= 1024) combine_norm_kernel<1><<<B, 256, 0, s>>>(y2, topk_w, inv_perm, out, H, k, norm_w, norm_out);
+    else if (H <= 2048) combine_norm_kernel<2><<<B, 256, 0, s>>>(y2, topk_w, inv_perm, out, H, k, norm_w, norm_out);
+    else if (H <= 3072) combine_norm_kernel<3><<<B, 256, 0, s>>>(y2, topk_w, inv_perm, out, H, k, norm_w, norm_out);
+    else combine_norm_kernel<4><<<B, 256, 0, s>>>(y2, topk_w, inv_perm, out, H, k, norm_w, norm_out);
+    GPTOSS_LAUNCH_CHECK("combine_norm_kernel");
+    return GPTOSS_OK;
+  }
   {
     TraceScope ts("combine", s);
     combine_kernel<<<B, 256, 0, s>>>(y2, topk_w, inv_perm, out, H, k, accumulate);

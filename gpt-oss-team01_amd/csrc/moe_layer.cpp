@@ -111,7 +111,7 @@ extern "C" int gptoss_moe_workspace_views(void *workspace, int B, int E, int k, 
 
 static int moe_forward_impl(const gptoss_moe_weights *w, const void *t, int B, float *out,
                             int accumulate, void *workspace, size_t workspace_bytes, void *stream,
-                            int mxfp4) {
+                            int mxfp4, const float *norm_w = nullptr, bf16_t *norm_out = nullptr) {
   int rc = check_moe(w, t, B, out, workspace, workspace_bytes);
   if (rc != GPTOSS_OK) return rc;
   if (B == 0) return GPTOSS_OK;
@@ -160,7 +160,13 @@ static int moe_forward_impl(const gptoss_moe_weights *w, const void *t, int B, f
   rc = run_gemm(g2, false, EPI_F32, rpt, max_tiles, s);
   if (rc != GPTOSS_OK) return rc;
 
-  return run_combine(ws.y2, ws.topk_w, ws.inv_perm, out, B, H, k, accumulate, s);
+  return run_combine(ws.y2, ws.topk_w, ws.inv_perm, out, B, H, k, accumulate, norm_w, norm_out, s);
+}
+
+int gptoss::moe_forward_norm(const gptoss_moe_weights *w, const void *t, int B, float *out, void *workspace,
+                             size_t workspace_bytes, hipStream_t s, int mxfp4, const float *norm_w,
+                             bf16_t *norm_out) {
+  return moe_forward_impl(w, t, B, out, 1, workspace, workspace_bytes, s, mxfp4, norm_w, norm_out);
 }
 
 extern "C" int gptoss_moe_forward(const gptoss_moe_weights *w, const void *t, int B, float *out,
