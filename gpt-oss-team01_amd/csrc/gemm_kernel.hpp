@@ -280,7 +280,9 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, bf16_t *lds, int 
     }
     // af[0] already holds the fragments of k-step 0 (requested before the previous barrier).  The
     // fragments of k-step kk+1 are requested before the MFMAs of k-step kk are issued, and the
-    // scheduling fences keep the compiler from sinking those reads next to their uses.
+    // scheduling fences keep the compiler from sinking those reads next to their uses (bf16; with
+    // MXFP4 weights the compiler is left free to weave the operand expansion between the MFMAs,
+    // measured 2 % faster).
 #pragma unroll
     for (int kk = 0; kk < 4; kk++) {
       if (kk + 1 < 4) {
@@ -292,11 +294,11 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, bf16_t *lds, int 
       bf16x8 b;
       if (FP4) b = as_bf16x8(fp4_expand(ring.b[R][0][kk], scale[kk >> 1]));
       else b = as_bf16x8(ring.b[R][kk % BQ]);
-      __builtin_amdgcn_sched_barrier(0);
+      if (!FP4) __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int i = 0; i < MB; i++)
         acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b, af[kk & 1][i], acc[i], 0, 0, 0);
-      __builtin_amdgcn_sched_barrier(0);
+      if (!FP4) __builtin_amdgcn_sched_barrier(0);
     }
   };
   auto read_first_frags = [&](int stage) {
