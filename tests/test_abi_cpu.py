@@ -94,3 +94,38 @@ def test_getp_hooks_compile_inside_the_reference_tu():
            "g++ -std=c++17 -fsyntax-only -w -x c++ - -I%s -I%s/include" % (REF, include, REF, REF, ROOT))
     r = subprocess.run(["bash", "-c", cmd], capture_output=True, text=True)
     assert r.returncode == 0, r.stderr[-2000:]
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py is a one-GPU benchmark: --gpus N with N > 1 (or a multi-rank launch) exits with a
+    message instead of running, before anything touches a device."""
+    import sys
+    for extra_env, args in (({}, ["--gpus", "2"]), ({"WORLD_SIZE": "2"}, [])):
+        r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py")] + args, capture_output=True, text=True,
+                           env=dict(os.environ, **extra_env), timeout=120)
+        assert r.returncode == 2, (r.returncode, r.stderr[-300:])
+        assert "ONE GPU" in r.stderr and r.stdout.strip() == ""
+
+
+def test_engine_entry_points_validate_before_touching_a_device(lib):
+    L = lib.load()
+    buf = (C.c_char * 256)()
+    p = C.cast(buf, C.c_void_p)
+    # null engine / null buffers
+    assert L.gptoss_engine_step(None, p, 0, 1, p) == 1
+    assert L.gptoss_engine_step_ragged(None, p, p, 1, p) == 1
+    assert L.gptoss_engine_prefill(None, p, 1, 1, p) == 1
+    n = C.c_longlong(0)
+    assert L.gptoss_engine_generate(None, p, p, 1, 1, 8, p, C.byref(n)) == 1
+    assert L.gptoss_engine_generate_ragged(None, p, p, 1, 1, 8, None, p, C.byref(n)) == 1
+    # prompt attention: shape checks come before any launch
+    assert L.gptoss_attn_prefill(p, p, p, None, p, 0, 4, 0, 8, 2, 32, 64, 0, p, 1 << 20, None) == 2      # B = 0
+    assert L.gptoss_attn_prefill(p, p, p, None, p, 1, 200, 0, 8, 2, 32, 128, 128, p, 1 << 20, None) == 2  # ring too short
+    assert "windowed cache" in lib.last_error()
+    assert L.gptoss_attn_prefill_workspace_bytes(0, 4, 8, 2, 32, 64) == 0
+    assert L.gptoss_attn_prefill_workspace_bytes(2, 64, 8, 2, 32, 64) > 2 * 64 * 4
+    # flags that exclude each other
+    cfg = lib.Config(4096, 256, 8, 4, 256, 4, 32, 8, 2, 64, 4096, 150000.0, 32.0, 128, 7.0)
+    h = C.c_void_p()
+    assert L.gptoss_engine_create(C.byref(cfg), p, 2, 16, lib.ENGINE_PRECISE | lib.ENGINE_SYNTHETIC, 0, C.byref(h)) == 6
+    assert L.gptoss_engine_create(C.byref(cfg), p, 2, 16, lib.ENGINE_PRECISE | lib.ENGINE_MXFP4_EXPERTS, 0, C.byref(h)) == 6

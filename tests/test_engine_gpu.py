@@ -408,3 +408,43 @@ def test_mxfp4_expert_storage_is_bit_identical_to_bf16_storage(ops, orc, tiny, s
     with pytest.raises(lib.GptossError) as ei:
         ops.Engine(cfg, tiny[2], max_batch=2, max_seq=16, mxfp4_experts=True)
     assert ei.value.code == 6 or "MXFP4" in str(ei.value)
+
+
+def test_prefill_and_ragged_step_edge_cases(ops, tiny):
+    """One position, one sequence, the whole context in one pass; arguments out of range."""
+    from conftest import load_pkg
+    lib = load_pkg("lib")
+    fx, cfg, flat = tiny
+    prompts = np.asarray(fx["prompts"], np.int32)
+    a = ops.Engine(cfg, flat, max_batch=3, max_seq=32)
+    b = ops.Engine(cfg, flat, max_batch=3, max_seq=32)
+    # T = 1 is one lock-step step
+    assert np.array_equal(a.prefill(prompts[:3, :1]), b.step(prompts[:3, 0], 0))
+    assert np.array_equal(a.last_logits(3), b.last_logits(3))
+    # a single sequence, the whole context (T = max_seq) in one pass
+    na = a.prefill(prompts[5:6, :32])
+    for pos in range(32):
+        nb = b.step(prompts[5:6, pos], pos)
+    assert np.array_equal(na, nb) and np.array_equal(a.last_logits(1), b.last_logits(1))
+    # ragged step with equal positions is the lock-step step
+    a.step(prompts[:3, 0], 0), b.step(prompts[:3, 0], 0)
+    assert np.array_equal(a.step_ragged(prompts[:3, 1], [1, 1, 1]), b.step(prompts[:3, 1], 1))
+    assert np.array_equal(a.last_logits(3), b.last_logits(3))
+    wide = np.concatenate([prompts[:3], prompts[:3, :1]], axis=1)     # 33 positions
+    for bad in (lambda: a.prefill(wide),                              # more positions than max_seq
+                lambda: a.prefill(prompts[:4, :4]),                   # more sequences than max_batch
+                lambda: a.step_ragged(prompts[:3, 0], [0, 32, 0]),    # a position beyond max_seq
+                lambda: a.step_ragged(prompts[:3, 0], [0, -1, 0]),
+                lambda: a.generate(prompts[:3, :4], 40)):             # longer than the engine holds
+        with pytest.raises(lib.GptossError):
+            bad()
+    a.close()
+    b.close()
+    c = ops.Engine(cfg, flat, max_batch=2, max_seq=16, precise=True)
+    with pytest.raises(lib.GptossError):
+        c.step_ragged(prompts[:2, 0], [0, 0])
+    with pytest.raises(lib.GptossError):
+        c.prefill(prompts[:2, :4])
+    with pytest.raises(lib.GptossError):
+        c.generate(prompts[:2, :4], 12, max_len=[8, 8])              # limits need the continuous schedule
+    c.close()
