@@ -19,6 +19,8 @@ struct GemmParams {
   const int *tiles;    // {n_tiles, (mat,row0,rows)*} or nullptr for a dense problem
   const int *xcd_bounds;  // 9 positions in the tile list (tile << 16 | 16-bit fraction) that cut the
                           // work into 8 parts of equal estimated cost, or nullptr: equal item counts
+  int tile_block;      // grouped problems: row tiles that are walked together, column tile by column
+                       // tile (0 or 1 = every row tile on its own)
   int dense_rows;      // rows of the dense problem when tiles == nullptr
   int N, K;
   int n_col_tiles;     // gemm_col_tiles(N)

@@ -471,7 +471,18 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void grouped_gemm_kernel(GemmParam
     const int work = lo + jj;
     Item it;
     int tile;
-    if (p.tiles) {
+    if (p.tiles && p.tile_block > 1) {
+      // grouped, experts with several row tiles: blocks of tile_block consecutive row tiles (mostly
+      // one expert's) are walked column tile by column tile, so that the workgroups of an XCD
+      // share each W column tile among the block's row tiles as well as each row tile among a
+      // few column tiles
+      const int per_block = p.tile_block * p.n_col_tiles;
+      const int tb = work / per_block;
+      const int v = work - tb * per_block;
+      const int th = min(p.tile_block, n_tiles - tb * p.tile_block);
+      it.ct = v / th;
+      tile = tb * p.tile_block + (v - it.ct * th);
+    } else if (p.tiles) {
       // grouped: column tiles of one row tile are neighbours (the tile's gathered rows stay in L2)
       tile = work / p.n_col_tiles;
       it.ct = work - tile * p.n_col_tiles;
