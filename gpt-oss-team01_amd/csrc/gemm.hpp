@@ -27,7 +27,7 @@ struct GemmParams {
   float limit;         // SwiGLU clamp
 };
 
-// rows_per_tile in {32,64,96,128,160} (96 only without gather); max_tiles bounds the number of
+// rows_per_tile in {32,64,96,128,160}; max_tiles bounds the number of
 // (mat,row-tile) items.
 int run_gemm(const GemmParams &p, bool gather, int epi, int rows_per_tile, int max_tiles,
              hipStream_t s);

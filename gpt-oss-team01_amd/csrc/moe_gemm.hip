@@ -204,8 +204,7 @@ static int dispatch_rows(const GemmParams &p, int rows_per_tile, int max_tiles, 
     case 32: return q ? launch_gemm<1, GATHER, EPI, true>(p, max_tiles, s) : launch_gemm<1, GATHER, EPI, false>(p, max_tiles, s);
     case 64: return q ? launch_gemm<2, GATHER, EPI, true>(p, max_tiles, s) : launch_gemm<2, GATHER, EPI, false>(p, max_tiles, s);
     case 96:
-      if constexpr (!GATHER) return q ? launch_gemm<3, GATHER, EPI, true>(p, max_tiles, s) : launch_gemm<3, GATHER, EPI, false>(p, max_tiles, s);
-      break;
+      return q ? launch_gemm<3, GATHER, EPI, true>(p, max_tiles, s) : launch_gemm<3, GATHER, EPI, false>(p, max_tiles, s);
     case 128: return q ? launch_gemm<4, GATHER, EPI, true>(p, max_tiles, s) : launch_gemm<4, GATHER, EPI, false>(p, max_tiles, s);
     case 160: return q ? launch_gemm<5, GATHER, EPI, true>(p, max_tiles, s) : launch_gemm<5, GATHER, EPI, false>(p, max_tiles, s);
   }
