@@ -100,6 +100,9 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
   const int n = lane & 15, c = lane >> 4;
   const int G = p.G;
   const int head = g * G + min(n, G - 1);
+  // the head's sink logit is only needed by the epilogue; requested here, its latency is hidden
+  // behind the whole pass instead of sitting between the last block and the output store
+  const float sink_logit = p.sinks ? p.sinks[head] : -INFINITY;
 
   const int seq = (p.rows_per_seq > 1) ? b / p.rows_per_seq : b;
   const bf16_t *kbase = p.kc + ((size_t)(seq * p.n_kv + g) * p.cap) * D;
@@ -244,15 +247,14 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
     else process(blk, buf, std::false_type{});
   };
 
-  const int last_blk = max(c0, ((c1 - 1) & ~(ATT_BLOCK - 1)));
   if (c1 > c0) {
     int blk = c0;
     while (true) {
-      load_kv(min(blk + ATT_BLOCK, last_blk), R1{});
+      if (blk + ATT_BLOCK < c1) load_kv(blk + ATT_BLOCK, R1{});  // wave-uniform: no reload of the last block
       step(blk, R0{});
       blk += ATT_BLOCK;
       if (blk >= c1) break;
-      load_kv(min(blk + ATT_BLOCK, last_blk), R0{});
+      if (blk + ATT_BLOCK < c1) load_kv(blk + ATT_BLOCK, R0{});
       step(blk, R1{});
       blk += ATT_BLOCK;
       if (blk >= c1) break;
@@ -265,7 +267,7 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
   if (n >= G) return;
   const int hq = g * G + n;
   if (r.nchunks == 1) {
-    float sink2 = p.sinks ? p.sinks[hq] * 1.4426950408889634f : -INFINITY;
+    float sink2 = sink_logit * 1.4426950408889634f;  // lanes that get here have head == hq
     float M = fmaxf(m_run, sink2);
     float w = exp2f(m_run - M);
     float denom = l_run * w + exp2f(sink2 - M);
