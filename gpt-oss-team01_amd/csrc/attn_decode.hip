@@ -241,8 +241,12 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
       }
   };
   const bool wrapped = r.len > p.cap;
+  // a wrapped ring no longer than the window (the engine's window layers) holds active positions
+  // in every slot: nothing to mask
+  const bool ring_all_active = wrapped && (p.window <= 0 || p.window >= p.cap);
   auto step = [&](int blk, auto buf) {
-    const bool edge = wrapped || blk < r.t_lo || blk + ATT_BLOCK > c1;  // wave-uniform
+    // wave-uniform (r.t_lo is a position: comparable with a slot index only while the ring has not wrapped)
+    const bool edge = blk + ATT_BLOCK > c1 || (!ring_all_active && (wrapped || blk < r.t_lo));
     if (edge) process(blk, buf, std::true_type{});
     else process(blk, buf, std::false_type{});
   };
