@@ -73,7 +73,13 @@ __device__ __forceinline__ SeqRange seq_range(int len, int cap, int window, int 
   return r;
 }
 
-template <int D>
+// PAIR (prompt passes, at most 8 query heads per kv head, ring not wrapped): a wave serves two
+// consecutive query rows of one sequence, row b in operand columns 0-7 and row b+1 in columns 8-15,
+// from one pass over the K/V blocks either of them needs.  Columns are independent in both MFMAs
+// and a block outside a row's own range is a no-op for its columns (scores -inf: max unchanged,
+// rescale factor exactly 1, probabilities exactly 0), so each row's result equals that of the
+// one-row kernel bit for bit.
+template <int D, bool PAIR>
 __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
   constexpr int KS = D / 32;   // k-steps of the score MFMA
   constexpr int DB = D / 16;   // 16-row blocks of O^T
@@ -82,24 +88,43 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
   const int item = blockIdx.x * 4 + wave;  // wave-uniform: everything derived from it stays scalar
   const int g = item % p.n_kv;
   const int rest = item / p.n_kv;
-  const int b = rest % p.B;
+  // work units per kv head and chunk: rows, or pairs of rows formed inside each sequence
+  // (rows_per_seq odd: the last row of a sequence is a pair of one)
+  const int pairs_per_seq = (p.rows_per_seq + 1) >> 1;
+  const int units = PAIR ? (p.B / p.rows_per_seq) * pairs_per_seq : p.B;
+  const int unit = rest % units;
+  const int pair_seq = unit / pairs_per_seq, pair_idx = unit - pair_seq * pairs_per_seq;
+  const int b = PAIR ? pair_seq * p.rows_per_seq + 2 * pair_idx : unit;
   // late chunks first: only long sequences have them, so the sparse part of the grid runs while
   // the chip is still filling and the grid ends on chunk 0, which every sequence has
-  const int chunk_id = p.max_chunks - 1 - rest / p.B;
+  const int chunk_id = p.max_chunks - 1 - rest / units;
   if (chunk_id < 0) return;
   const SeqRange r = seq_range(__builtin_amdgcn_readfirstlane(p.lens[b]), p.cap, p.window, p.max_len);
-  if (chunk_id >= r.nchunks) return;
+  // the second row of a pair: the next row of the same sequence, when there is one
+  const bool two = PAIR && 2 * pair_idx + 1 < p.rows_per_seq;
+  const SeqRange r1 = two ? seq_range(__builtin_amdgcn_readfirstlane(p.lens[b + 1]), p.cap, p.window, p.max_len) : r;
+  const bool act0 = chunk_id < r.nchunks, act1 = two && chunk_id < r1.nchunks;
+  if (!act0 && !act1) return;
   // position held by slot s is s + pos_base, or cap less when that would lie beyond the last one
   const int pos_base = (r.len > 0) ? ((r.len - 1) / p.cap) * p.cap : 0;
   auto slot_pos = [&](int s) {
     int pp = s + pos_base;
     return (pp > r.len - 1) ? pp - p.cap : pp;   // negative for a slot that was never written
   };
-  const int c0 = r.s_begin + chunk_id * r.chunk;
-  const int c1 = min(r.s_end, c0 + r.chunk);
+  // slot range of this chunk for each row ([0,0) for a row that has no such chunk), their active
+  // parts [lo, hi) (PAIR: slot == position), and the union the wave walks
+  const int c0_0 = r.s_begin + chunk_id * r.chunk, c0_1 = r1.s_begin + chunk_id * r1.chunk;
+  const int hi0 = act0 ? min(r.s_end, c0_0 + r.chunk) : 0, hi1 = act1 ? min(r1.s_end, c0_1 + r1.chunk) : 0;
+  const int lo0 = max(c0_0, r.t_lo), lo1 = max(c0_1, r1.t_lo);
+  const int c0 = !PAIR ? c0_0 : (act0 && act1) ? min(c0_0, c0_1) : act0 ? c0_0 : c0_1;
+  const int c1 = !PAIR ? hi0 : max(hi0, hi1);
   const int n = lane & 15, c = lane >> 4;
   const int G = p.G;
-  const int head = g * G + min(n, G - 1);
+  const bool second = PAIR && n >= 8;            // lane's operand column belongs to row b+1
+  const int hn = PAIR ? (n & 7) : n;             // head within the kv group
+  const bool col_live = hn < G && (!second || two);
+  const int bn = (second && two) ? b + 1 : b;    // the column's query row
+  const int head = g * G + min(hn, G - 1);
   // the head's sink logit is only needed by the epilogue; requested here, its latency is hidden
   // behind the whole pass instead of sitting between the last block and the output store
   const float sink_logit = p.sinks ? p.sinks[head] : -INFINITY;
@@ -136,13 +161,13 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
   // ---- Q^T operand, split into bf16 hi and lo parts -----------------------------------------
   bf16x8 qh[KS], ql[KS];
   {
-    const float *qp = p.q + ((size_t)b * p.n_q + head) * D + c * KS * 8;
+    const float *qp = p.q + ((size_t)bn * p.n_q + head) * D + c * KS * 8;
 #pragma unroll
     for (int s = 0; s < KS; s++) {
       uint32_t h[4], l[4];
 #pragma unroll
       for (int j = 0; j < 4; j++) {
-        float x0 = (n < G) ? qp[s * 8 + 2 * j] : 0.f, x1 = (n < G) ? qp[s * 8 + 2 * j + 1] : 0.f;
+        float x0 = col_live ? qp[s * 8 + 2 * j] : 0.f, x1 = col_live ? qp[s * 8 + 2 * j + 1] : 0.f;
         bf16_t h0 = f32_to_bf16(x0), h1 = f32_to_bf16(x1);
         h[j] = (uint32_t)h0 | ((uint32_t)h1 << 16);
         l[j] = pack_bf16x2(x0 - bf16_to_f32(h0), x1 - bf16_to_f32(h1));
@@ -156,6 +181,8 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
 #pragma unroll
   for (int db = 0; db < DB; db++) o[db] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m_run = NEG_BIG, l_run = 0.f;
+
+  const int lane_lo = second ? lo1 : lo0, lane_hi = second ? hi1 : hi0;  // PAIR: the column's active slots
 
   // EDGE = the block holds slots outside the active positions (first/last block of a range, or
   // any block of a wrapped ring): only that variant carries the masking code.
@@ -181,9 +208,13 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
 #pragma unroll
       for (int i = 0; i < 4; i++) {
         float v = s4[tb][i] * p.scale_log2e;
+        // keep the product a rounded value of its own in both variants of this block (the unmasked
+        // one would otherwise fuse it into the subtraction below): a row's result must not depend
+        // on which variant its partner row forces
+        asm volatile("" : "+v"(v));
         if (EDGE) {
           const int slot = blk + tb * 16 + c * 4 + i;
-          const bool ok = slot < c1 && slot_pos(slot) >= r.t_lo;
+          const bool ok = PAIR ? (slot >= lane_lo && slot < lane_hi) : (slot < c1 && slot_pos(slot) >= r.t_lo);
           v = ok ? v : -INFINITY;
         }
         s4[tb][i] = v;
@@ -230,8 +261,11 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
 #pragma unroll
           for (int w = 0; w < 4; w++) {
             const int s_lo = blk + grp * 32 + (w >> 1) * 16 + c * 4 + (w & 1) * 2;
-            const uint32_t keep = ((s_lo < c1 && slot_pos(s_lo) >= r.t_lo) ? 0x0000ffffu : 0u) |
-                                  ((s_lo + 1 < c1 && slot_pos(s_lo + 1) >= r.t_lo) ? 0xffff0000u : 0u);
+            // PAIR: V rows are shared by the two rows' columns, a slot is kept if either row uses it
+            auto used = [&](int sl) {
+              return PAIR ? ((sl >= lo0 && sl < hi0) || (sl >= lo1 && sl < hi1)) : (sl < c1 && slot_pos(sl) >= r.t_lo);
+            };
+            const uint32_t keep = (used(s_lo) ? 0x0000ffffu : 0u) | (used(s_lo + 1) ? 0xffff0000u : 0u);
             vv[w] &= keep;
           }
         }
@@ -246,7 +280,8 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
   const bool ring_all_active = wrapped && (p.window <= 0 || p.window >= p.cap);
   auto step = [&](int blk, auto buf) {
     // wave-uniform (r.t_lo is a position: comparable with a slot index only while the ring has not wrapped)
-    const bool edge = blk + ATT_BLOCK > c1 || (!ring_all_active && (wrapped || blk < r.t_lo));
+    const bool edge = PAIR ? !(two && blk >= lo0 && blk + ATT_BLOCK <= hi0 && blk >= lo1 && blk + ATT_BLOCK <= hi1)
+                           : (blk + ATT_BLOCK > c1 || (!ring_all_active && (wrapped || blk < r.t_lo)));
     if (edge) process(blk, buf, std::true_type{});
     else process(blk, buf, std::false_type{});
   };
@@ -268,15 +303,17 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
   // ---- per-head totals: sum the partial denominators of the 4 lanes that share a head --------
   l_run += __shfl_xor(l_run, 16, 64);
   l_run += __shfl_xor(l_run, 32, 64);
-  if (n >= G) return;
-  const int hq = g * G + n;
-  if (r.nchunks == 1) {
+  if (!col_live) return;
+  if (PAIR && !(second ? act1 : act0)) return;  // this row has no such chunk
+  const int hq = g * G + hn;
+  const int row_chunks = second ? r1.nchunks : r.nchunks;
+  if (row_chunks == 1) {
     float sink2 = sink_logit * 1.4426950408889634f;  // lanes that get here have head == hq
     float M = fmaxf(m_run, sink2);
     float w = exp2f(m_run - M);
     float denom = l_run * w + exp2f(sink2 - M);
     float inv = (denom > 0.f) ? w / denom : 0.f;
-    bf16_t *op = p.out + ((size_t)b * p.n_q + hq) * D;
+    bf16_t *op = p.out + ((size_t)bn * p.n_q + hq) * D;
 #pragma unroll
     for (int db = 0; db < DB; db++) {
       u32x2 pk = u32x2{pack_bf16x2(o[db][0] * inv, o[db][1] * inv),
@@ -284,7 +321,7 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
       *reinterpret_cast<u32x2 *>(op + db * 16 + c * 4) = pk;
     }
   } else {
-    const size_t slot = ((size_t)b * p.max_chunks + chunk_id) * p.n_q + hq;
+    const size_t slot = ((size_t)bn * p.max_chunks + chunk_id) * p.n_q + hq;
     float *po = p.part_o + slot * D;
 #pragma unroll
     for (int db = 0; db < DB; db++) *reinterpret_cast<f32x4 *>(po + db * 16 + c * 4) = o[db];
@@ -473,12 +510,20 @@ static int attn_launch(const float *q, const void *k_cache, const void *v_cache,
   p.max_len = max_len;
   p.scale_log2e = 1.4426950408889634f / sqrtf((float)head_dim);
   hipStream_t s = (hipStream_t)stream;
-  long long items = (long long)B * n_kv * pl.max_chunks;
+  // prompt passes put two consecutive rows of a sequence into one wave when the 16 operand columns
+  // hold both rows' query heads and no ring can have wrapped (slot == position)
+  const bool pair = rows_per_seq > 1 && B % rows_per_seq == 0 && p.G <= 8 && max_len <= capacity;
+  long long items = (long long)(pair ? (B / rows_per_seq) * ((rows_per_seq + 1) / 2) : B) * n_kv * pl.max_chunks;
   int grid = (int)((items + 3) / 4);
   {
     TraceScope ts("attn_decode", s);
-    if (head_dim == 64) attn_decode_kernel<64><<<grid, 256, 0, s>>>(p);
-    else attn_decode_kernel<32><<<grid, 256, 0, s>>>(p);
+    if (head_dim == 64) {
+      if (pair) attn_decode_kernel<64, true><<<grid, 256, 0, s>>>(p);
+      else attn_decode_kernel<64, false><<<grid, 256, 0, s>>>(p);
+    } else {
+      if (pair) attn_decode_kernel<32, true><<<grid, 256, 0, s>>>(p);
+      else attn_decode_kernel<32, false><<<grid, 256, 0, s>>>(p);
+    }
   }
   GPTOSS_LAUNCH_CHECK("attn_decode_kernel");
   if (pl.max_chunks > 1) {

@@ -169,6 +169,9 @@ def test_attn_batch_larger_than_one_launch_slice(ops, orc):
     (2, 300, 0, 64, 8, 64, 128),      # prompt longer than the window (linear cache)
     (2, 70, 500, 64, 8, 64, 0),       # a later slice of a long context: two chunks per row
     (1, 200, 1000, 64, 8, 64, 0),     # rows on both sides of the 1024-position chunk-size change
+    (2, 65, 60, 64, 8, 64, 128),      # odd row count (the last row of a sequence has no partner), window edges
+    (3, 41, 0, 8, 2, 32, 0),          # odd row count, four query heads per kv head
+    (1, 66, 480, 64, 8, 64, 0),       # partners on either side of a chunk boundary (512 / 513 positions)
 ])
 def test_attn_prefill_rows_equal_decode_calls(ops, orc, B, T, pos0, n_q, n_kv, D, window):
     """Prompt attention = the decode attention of every position at once: row (b, t) must equal, bit
@@ -190,7 +193,8 @@ def test_attn_prefill_rows_equal_decode_calls(ops, orc, B, T, pos0, n_q, n_kv, D
     torch.cuda.synchronize()
     assert torch.isfinite(got.float()).all()
     dec = ops.AttnDecode(B, n_q, n_kv, D, S)
-    for t in sorted({0, 1, T // 3, T // 2, T - 2, T - 1}):
+    # every row of the short prompts (two consecutive rows share a wave), a sample of the long ones
+    for t in (range(T) if T <= 70 else sorted({0, 1, T // 3, T // 2, T - 2, T - 1})):
         lens = torch.full((B,), pos0 + t + 1, dtype=torch.int32)
         one = dec.forward(q[:, t].contiguous().cuda(), cache, lens.cuda(), sinks.cuda(), window=window,
                           max_len=pos0 + t + 1)
