@@ -17,7 +17,8 @@
 //     The chunk length is a constant, so a row's result is the same whatever else is in the
 //     launch;
 //   * several query rows may share one sequence's cache (rows_per_seq), each with its own length:
-//     the T positions of a prompt are T such rows, which is all the prompt-pass attention is.
+//     the T positions of a prompt are T such rows, which is all the prompt-pass attention is; two
+//     consecutive rows of a sequence then share a wave (8 heads each in the 16 operand columns).
 #include <algorithm>
 #include <type_traits>
 
