@@ -270,7 +270,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, bf16_t *lds, int 
 
   const bf16_t *a_src = lds + (lane & 31) * LDS_ROW + (lane >> 5) * 8;
   bf16x8 af[2][MB];
-  auto compute = [&](int stage, auto rsel) {
+  auto compute = [&](int stage, auto rsel, auto &&after_kstep) {
     constexpr int R = decltype(rsel)::value;
     const bf16_t *base = a_src + stage * LDS_STAGE;
     float scale[2] = {0.f, 0.f};  // of k 0-31 and k 32-63 of the slab
@@ -298,6 +298,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, bf16_t *lds, int 
 #pragma unroll
       for (int i = 0; i < MB; i++)
         acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b, af[kk & 1][i], acc[i], 0, 0, 0);
+      after_kstep(kk);
       if (!FP4) __builtin_amdgcn_sched_barrier(0);
     }
   };
@@ -342,8 +343,22 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, bf16_t *lds, int 
     // then the first slabs of the next item
     const int t = s + D;
     const bool wrap = t >= padded;
-    w_load<NRING, FP4>(ring, wrap ? next : cur, min(wrap ? t - padded : t, last), lane, Refill{});
-    compute(st, rsel);
+    const WStream &wsrc = wrap ? next : cur;
+    const int wslab = min(wrap ? t - padded : t, last);
+    // Without the token gather (dense GEMMs, GEMM2) each of the refill slab's four 1 KB fragments
+    // is requested right after the MFMAs of one k-step, so issuing it costs no time of its own
+    // (classifier -4 %, projections of a prompt pass -3 %); GEMM1 keeps all four requests at the
+    // top of the iteration, where its HBM-bound stream measured 2 % faster.
+    constexpr bool W_PER_KSTEP = !FP4 && !GATHER;
+    if constexpr (!W_PER_KSTEP) {
+      w_load<NRING, FP4>(ring, wsrc, wslab, lane, Refill{});
+      compute(st, rsel, [](int) {});
+    } else {
+      compute(st, rsel, [&](int kk) {
+        ring.b[Refill::value][kk % BQ] =
+            *reinterpret_cast<const u32x4 *>(wsrc.w + (size_t)(wslab * 4 + kk) * 512 + lane * 8);
+      });
+    }
     const int st1 = (st == 2) ? 0 : st + 1, st2 = (st1 == 2) ? 0 : st1 + 1;
     store_a(st2, s + 2 >= nslab, psel);  // rows of slab s+2 (zeros while padding)
     load_a(min(s + 2 + APF, last), psel);
