@@ -270,19 +270,22 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, bf16_t *lds, int 
 
   const bf16_t *a_src = lds + (lane & 31) * LDS_ROW + (lane >> 5) * 8;
   bf16x8 af[2][MB];
-  auto compute = [&](int stage, auto rsel, auto &&after_kstep) {
+  auto compute = [&](int stage, int next_stage, auto rsel, auto &&after_kstep) {
     constexpr int R = decltype(rsel)::value;
     const bf16_t *base = a_src + stage * LDS_STAGE;
+    const bf16_t *nbase = a_src + next_stage * LDS_STAGE;
     float scale[2] = {0.f, 0.f};  // of k 0-31 and k 32-63 of the slab
     if (FP4) {
       scale[0] = fp4_scale(ring.s[R] & 0xffu);
       scale[1] = fp4_scale((ring.s[R] >> 8) & 0xffu);
     }
     // af[0] already holds the fragments of k-step 0 (requested before the previous barrier).  The
-    // fragments of k-step kk+1 are requested before the MFMAs of k-step kk are issued, and the
-    // scheduling fences keep the compiler from sinking those reads next to their uses (bf16; with
-    // MXFP4 weights the compiler is left free to weave the operand expansion between the MFMAs,
-    // measured 2 % faster).
+    // fragments of k-step kk+1 are requested before the MFMAs of k-step kk are issued (bf16: before
+    // those of the last k-step, the first fragments of the next slab, whose stage is complete since
+    // the previous barrier), and the scheduling fences keep the compiler from sinking those reads
+    // next to their uses (bf16; with MXFP4 weights the compiler is left free to weave the operand
+    // expansion between the MFMAs, measured 2 % faster).  after_kstep(kk) is what else the iteration
+    // has to issue, placed behind the MFMAs of a k-step so that it costs no time of its own.
 #pragma unroll
     for (int kk = 0; kk < 4; kk++) {
       if (kk + 1 < 4) {
@@ -290,6 +293,10 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, bf16_t *lds, int 
         for (int i = 0; i < MB; i++)
           af[(kk + 1) & 1][i] =
               as_bf16x8(*reinterpret_cast<const u32x4 *>(base + i * 32 * LDS_ROW + (kk + 1) * 16));
+      } else if (!FP4) {
+#pragma unroll
+        for (int i = 0; i < MB; i++)
+          af[0][i] = as_bf16x8(*reinterpret_cast<const u32x4 *>(nbase + i * 32 * LDS_ROW));
       }
       bf16x8 b;
       if (FP4) b = as_bf16x8(fp4_expand(ring.b[R][0][kk], scale[kk >> 1]));
@@ -345,24 +352,29 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, bf16_t *lds, int 
     const bool wrap = t >= padded;
     const WStream &wsrc = wrap ? next : cur;
     const int wslab = min(wrap ? t - padded : t, last);
-    // Without the token gather (dense GEMMs, GEMM2) each of the refill slab's four 1 KB fragments
-    // is requested right after the MFMAs of one k-step, so issuing it costs no time of its own
-    // (classifier -4 %, projections of a prompt pass -3 %); GEMM1 keeps all four requests at the
-    // top of the iteration, where its HBM-bound stream measured 2 % faster.
+    const int st1 = (st == 2) ? 0 : st + 1, st2 = (st1 == 2) ? 0 : st1 + 1;
+    // bf16: everything the iteration issues besides MFMAs and fragment reads sits behind the MFMAs
+    // of a k-step.  Without the token gather (dense GEMMs, GEMM2) each of the refill slab's four
+    // 1 KB fragments is requested after one k-step (classifier -6 %, projections of a prompt pass
+    // -5 %); GEMM1 keeps all four requests at the top of the iteration, where its HBM-bound stream
+    // measured 2 % faster.  The rows of slab s+2 go to LDS after k-step 1 and the next rows are
+    // requested after k-step 2 (GEMM1 of a prompt pass -5 %; after k-steps 0 and 1: no gain).
     constexpr bool W_PER_KSTEP = !FP4 && !GATHER;
-    if constexpr (!W_PER_KSTEP) {
-      w_load<NRING, FP4>(ring, wsrc, wslab, lane, Refill{});
-      compute(st, rsel, [](int) {});
-    } else {
-      compute(st, rsel, [&](int kk) {
+    if constexpr (!W_PER_KSTEP) w_load<NRING, FP4>(ring, wsrc, wslab, lane, Refill{});
+    compute(st, st1, rsel, [&](int kk) {
+      if constexpr (W_PER_KSTEP)
         ring.b[Refill::value][kk % BQ] =
             *reinterpret_cast<const u32x4 *>(wsrc.w + (size_t)(wslab * 4 + kk) * 512 + lane * 8);
-      });
+      if constexpr (!FP4) {
+        if (kk == 1) store_a(st2, s + 2 >= nslab, psel);  // rows of slab s+2 (zeros while padding)
+        if (kk == 2) load_a(min(s + 2 + APF, last), psel);
+      }
+    });
+    if constexpr (FP4) {
+      store_a(st2, s + 2 >= nslab, psel);
+      load_a(min(s + 2 + APF, last), psel);
+      read_first_frags(st1);
     }
-    const int st1 = (st == 2) ? 0 : st + 1, st2 = (st1 == 2) ? 0 : st1 + 1;
-    store_a(st2, s + 2 >= nslab, psel);  // rows of slab s+2 (zeros while padding)
-    load_a(min(s + 2 + APF, last), psel);
-    read_first_frags(st1);
     st = st1;
     __syncthreads();
   };
