@@ -333,10 +333,19 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, bf16_t *lds, int 
     load_a(min(2, last), P0{});
     load_a(min(3, last), P1{});
   } else {
+    // slabs 0 and 1 are requested together (the second into registers that are only live here), so
+    // the prologue waits for one round trip to memory instead of two
+    u32x4 first[AC];
     load_a(0, P0{});
+#pragma unroll
+    for (int i = 0; i < AC; i++)
+      if (a_live[i]) first[i] = *reinterpret_cast<const u32x4 *>(p.A + a_off[i] + min(1, last) * BK);
     store_a(0, false, P0{});
-    load_a(min(1, last), P0{});
-    store_a(1, nslab <= 1, P0{});
+#pragma unroll
+    for (int i = 0; i < AC; i++)
+      if (a_live[i])
+        *reinterpret_cast<u32x4 *>(a_dst + LDS_STAGE + APASS * i * LDS_ROW) =
+            (nslab <= 1) ? u32x4{0u, 0u, 0u, 0u} : first[i];
     load_a(min(2, last), P0{});
   }
   __syncthreads();
