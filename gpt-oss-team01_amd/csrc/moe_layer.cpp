@@ -47,8 +47,9 @@ static MoeWorkspace carve(void *base, int B, int E, int k, int H, int I) {
 // and its weights are streamed exactly once; the kernel is bound by that stream.
 // MXFP4 weights (32, 64 or 96 rows): tiles of at most 96 rows, whose kernels run two workgroups
 // per CU; an expert's few row tiles are walked column tile by column tile (tile_block), so its
-// weights still come from HBM once.  64 rows up to ~200 rows per expert, 96 beyond (measured on
-// 32 experts from 256 to 8192 tokens: each choice within 5 % of the better one everywhere).
+// weights still come from HBM once.  96 rows only where they hold a whole expert; beyond that 64
+// (the 64-row kernel has room for a five-slab W ring, the 96-row one spills a few registers:
+// prompt passes of 8192 tokens 1.3 % faster with 64).
 int moe_rows_per_tile(int B, int k, int E, bool mxfp4) {
   double avg = (double)B * k / E;
   double need = avg + 2.5 * sqrt(avg);
@@ -56,8 +57,7 @@ int moe_rows_per_tile(int B, int k, int E, bool mxfp4) {
   if (need <= 32) return 32;
   if (need <= 64) return 64;
   if (mxfp4) {
-    if (need <= 96) return 96;
-    return avg < 224 ? 64 : 96;
+    return need <= 96 ? 96 : 64;
   }
   if (need <= 128) return 128;
   return 160;
