@@ -29,7 +29,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
 # HBM bytes of one GEMM1 launch at the default workload, from two rocprofv3 --pmc runs of this
 # command (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, the factors the 1 GiB copy below calibrates); the
 # summary is kept in profiles/moe_layer_20b_1024tok_and_decode_attention_kernel_stats_and_hbm_traffic.md
-GEMM1_HBM_TRAFFIC_BYTES = (1_103_482 + 23_041) * 1024
+GEMM1_HBM_TRAFFIC_BYTES = (1_101_846 + 23_041) * 1024
 
 
 def parse():
