@@ -5,7 +5,8 @@ plus what a test needs to rebuild the same checkpoint and prompts from seeds.
 
 Run in the build container (the reference tree is needed):
     make -C oracle ref && python tests/golden/make_golden.py
-The fixture holds data only: seeds, the checkpoint's SHA-256, prompts, expected ids, logit margins.
+The fixture holds data only: seeds, the checkpoint's SHA-256, prompts, expected ids, logit margins
+and router gaps.
 """
 import hashlib
 import importlib
@@ -46,6 +47,18 @@ def main():
         flat = np.fromfile(path, dtype="<f4", offset=binfmt.HEADER_BYTES)
         o_out, o_n, margins = orc.generate(cfg, flat, prompts, MAX_SEQ, want_margins=True)
         assert np.array_equal(ref_out, o_out) and ref_n == o_n, "oracle differs from the reference"
+        # per generated id: the smallest gap between the 4th and 5th router score over the layers of
+        # the forward call that produced it (how close that call came to routing to another expert)
+        gaps = np.zeros((N_REQ, N_GEN), np.float32)
+        for r in range(N_REQ):
+            m = orc.Model(cfg, flat)
+            seq = list(prompts[r]) + list(ref_out[r, :N_GEN])
+            for pos in range(MAX_SEQ - 1):
+                lg = m.forward(int(seq[pos]), pos)
+                if pos >= N_PROMPT - 1:
+                    assert int(lg.argmax()) == ref_out[r, pos - (N_PROMPT - 1)]
+                    gaps[r, pos - (N_PROMPT - 1)] = m.last_router_gap()
+            m.close()
         # first-step logits of request 0 from the reference itself
         import ctypes as C
         R = orc.ref()
@@ -63,6 +76,7 @@ def main():
         "min_logit_margin": float(margins[:, :N_GEN].min()),
         "min_router_gap": orc.generate.last_min_router_gap,
         "logit_margins": [[round(float(x), 6) for x in row[:N_GEN]] for row in margins],
+        "router_gaps": [[round(float(x), 6) for x in row] for row in gaps],
         "first_logits_req0": {"argmax": int(lg.argmax()), "max": float(lg.max()),
                               "sum": float(lg.astype(np.float64).sum()),
                               "head": [float(x) for x in lg[:8]]},

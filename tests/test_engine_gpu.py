@@ -95,26 +95,77 @@ def test_teacher_forced_ids_match_golden_where_margin_is_clear(ops, orc, tiny):
 
 
 def test_generate_follows_getp_loop_semantics(ops, orc, tiny):
-    """Free-running greedy generation: output layout, terminator and count as the harness expects;
-    ids equal to the CPU model run with the same bf16 staging for as long as its margins are clear,
-    and the prefix of agreement with the fp32 golden ids is reported."""
+    """Free-running greedy generation on the production (bf16-staged, MFMA) engine.
+
+    Layout, terminator and count are the harness's.  The ids cannot equal the fp32 golden ids
+    everywhere (top-1/top-2 logit margins and 4th/5th router gaps of this model reach 2e-4, below
+    the noise of six bf16 roundings per layer); what must hold instead, and is asserted:
+
+    1. every request's FIRST divergence from the golden ids sits at a position where the reference's
+       own decision is a near-tie: logit margin < 5e-3 or a router gap < 3e-3 in the forward call
+       that produced that id (both stored in the fixture; up to that position the engine has seen
+       exactly the golden history);
+    2. fed the engine's own output as history, the CPU model with the GPU dataflow's rounding points
+       (STAGE_GPU) picks the engine's id at every position that is not such a near-tie for it: the
+       engine's trajectory is a greedy trajectory of that model up to near-ties;
+    3. hence the STAGE_GPU model's free-running ids equal the engine's up to each request's first
+       near-tie position, which is checked directly as well.
+    """
     fx, cfg, flat = tiny
     prompts = np.asarray(fx["prompts"], np.int32)
     eng = ops.Engine(cfg, flat, max_batch=4, max_seq=fx["max_seq_len"])   # 8 requests, 2 batches
     out, n = eng.generate(prompts, fx["max_seq_len"])
     eng.close()
+    n_req, n_prompt = prompts.shape
     n_gen = fx["n_prompt"]
     assert n == fx["n_generated"]
     assert (out[:, fx["terminator_index"]] == -1).all()
     assert ((out[:, :n_gen] >= 0) & (out[:, :n_gen] < cfg.vocab_size)).all()
     gold = np.asarray(fx["expected_ids"], np.int32)
-    agree = (out[:, :n_gen] == gold)
-    first_diff = [int(np.argmin(a)) if not a.all() else n_gen for a in agree]
-    print("free-running agreement with the fp32 golden ids:", float(agree.mean()), first_diff)
-    # the first generated id of every request only depends on forced prompt tokens
     margins = np.asarray(fx["logit_margins"], np.float32)
-    clear0 = margins[:, 0] > 5e-3
-    assert (out[clear0, 0] == gold[clear0, 0]).all()
+    gaps = np.asarray(fx["router_gaps"], np.float32)
+    MARGIN, GAP = 5e-3, 3e-3
+
+    # 1. against the reference's fp32 ids
+    agree = out[:, :n_gen] == gold
+    first_diff = [int(np.argmin(a)) if not a.all() else n_gen for a in agree]
+    for r, d in enumerate(first_diff):
+        if d < n_gen:
+            assert margins[r, d] < MARGIN or gaps[r, d] < GAP, (r, d, float(margins[r, d]), float(gaps[r, d]))
+    print("free-running agreement with the fp32 golden ids:", float(agree.mean()), first_diff)
+
+    # 2. and 3. against the CPU model rounded where the GPU dataflow rounds
+    clear_total = pinned_total = 0
+    for r in range(n_req):
+        seq = np.concatenate([prompts[r], out[r, :n_gen]])
+        forced = orc.Model(cfg, flat, stage=orc.STAGE_GPU)       # sees the engine's history
+        free = orc.Model(cfg, flat, stage=orc.STAGE_GPU)         # feeds back its own ids
+        tok_free, free_alive = int(prompts[r, 0]), True
+        for pos in range(fx["max_seq_len"] - 1):
+            lg = forced.forward(int(seq[pos]), pos)
+            i = pos - (n_prompt - 1)
+            if free_alive:
+                lf = free.forward(tok_free, pos)
+                tok_free = int(prompts[r, pos + 1]) if i < 0 else int(lf.argmax())
+            if i < 0:
+                continue
+            top2 = np.partition(lg, -2)[-2:]
+            near = (top2[1] - top2[0]) < MARGIN or forced.last_router_gap() < GAP
+            if not near:
+                clear_total += 1
+                assert int(lg.argmax()) == out[r, i], (r, i, float(top2[1] - top2[0]), forced.last_router_gap())
+            if free_alive:
+                if near:
+                    free_alive = False          # from here on the two may legitimately part
+                else:
+                    pinned_total += 1
+                    assert tok_free == out[r, i], (r, i)
+        forced.close()
+        free.close()
+    print("positions where the staged CPU model's decision is clear:", clear_total, "of", n_req * n_gen,
+          "; ids pinned before each request's first near-tie:", pinned_total)
+    assert clear_total >= 0.6 * n_req * n_gen
+    assert pinned_total >= n_req                 # not vacuous: about one clear id per request at least
 
 
 def test_precise_engine_reproduces_the_golden_ids_exactly(ops, orc, tiny):

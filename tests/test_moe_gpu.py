@@ -196,3 +196,55 @@ def test_moe_forward_skewed_routing_is_batch_invariant(ops, orc, B, E, H, I):
     assert same.mean() > 0.9
     mx, mean = rel_errors(full.cpu().numpy()[:n_chk][same], want[same])
     assert mx <= TOL_MAX and mean <= TOL_MEAN, (mx, mean)
+
+
+# ---------------------------------------------------------------- SwiGLU epilogue and bias order, alone
+def test_swiglu_special_cases_and_bias_order_through_a_one_expert_layer(ops, orc):
+    """One expert, top-1, w2 = identity: the layer's output is the bf16-rounded clamped SwiGLU of
+    chosen (gate, up) values plus b2, so the epilogue of GEMM1 (run.cpp:669-686: gate = min(g, 7),
+    up = clamp(u, -7, 7), g * sigmoid(1.702 g) * (up + 1)), the (gate, up) interleave of mlp1's rows
+    and the order of both bias vectors are checked on their own, special cases included:
+    g > 7, u > 7, u < -7 (up + 1 = -6), g -> -inf (0)."""
+    H = I = 64
+    B = 4
+    gv = np.array([8.0, 7.0, 6.5, -100.0, 0.5, -0.5, 30.0, -8.0], np.float32)
+    uv = np.array([-8.0, 8.0, 0.25, 7.0, -7.0, -6.5, 100.0, -1.0], np.float32)
+    j = np.arange(I)
+    g_j, u_j = gv[j % 8], uv[(j // 8) % 8]
+    w1 = np.zeros((1, 2 * I, H), np.float32)
+    w1[0, 0::2, 0] = g_j                       # row 2j = gate of pair j, row 2j+1 = its up
+    w1[0, 1::2, 0] = u_j
+    b1 = np.zeros((1, 2 * I), np.float32)
+    b1[0, 0::2] = 0.125 * (j % 3)
+    b1[0, 1::2] = -0.25 * (j % 5)
+    b2 = (0.5 * (j % 7) - 1.0).astype(np.float32)[None]
+    w2 = np.eye(H, I, dtype=np.float32)[None]
+    s = np.array([1.0, 0.5, -1.0, 2.0], np.float32)
+    t = np.zeros((B, H), np.float32)
+    t[:, 0] = s
+    t[:, 5] = 3.0                              # a column no weight reads
+    tt = lambda a: torch.from_numpy(a).to(torch.bfloat16).cuda()
+    mk = lambda bias2: ops.MoeLayer(torch.zeros(1, H, dtype=torch.bfloat16).cuda(), torch.zeros(1).cuda(), tt(w1),
+                                    torch.from_numpy(b1).cuda(), tt(w2), torch.from_numpy(bias2).cuda(), top_k=1,
+                                    max_tokens=B)
+    got = mk(np.zeros_like(b2)).forward(tt(t)).cpu().numpy()
+    with_b2 = mk(b2).forward(tt(t)).cpu().numpy()
+    np.testing.assert_allclose(with_b2 - got, np.broadcast_to(b2, got.shape), atol=1e-5)   # b2[j] lands on column j
+    gate = s[:, None] * g_j[None, :] + b1[0, 0::2][None, :]
+    up = s[:, None] * u_j[None, :] + b1[0, 1::2][None, :]
+    pre = np.empty((B, 2 * I), np.float32)
+    pre[:, 0::2], pre[:, 1::2] = gate, up
+    want = orc.swiglu(pre, 7.0)
+    # closed form in float64, independent of the oracle
+    gc_, uc_ = np.minimum(gate.astype(np.float64), 7.0), np.clip(up.astype(np.float64), -7.0, 7.0)
+    closed = gc_ / (1.0 + np.exp(-1.702 * gc_)) * (uc_ + 1.0)
+    np.testing.assert_allclose(want, closed, rtol=1e-5, atol=1e-30)
+    # the GPU result is bf16-rounded (2^-9 relative) after exp2/reciprocal of a few ulp
+    np.testing.assert_allclose(got, closed, rtol=5e-3, atol=1e-30)
+    # the special cases, by value
+    big_g = gate > 7.0
+    assert big_g.any() and (up < -7.0).any() and (up > 7.0).any() and (gate < -50).any()
+    sig7 = 7.0 / (1.0 + np.exp(-1.702 * 7.0))
+    np.testing.assert_allclose(got[big_g], (sig7 * (uc_ + 1.0))[big_g], rtol=5e-3)
+    np.testing.assert_allclose(got[big_g & (up < -7.0)], sig7 * -6.0, rtol=5e-3)
+    assert (got[gate < -50] == 0).all()
