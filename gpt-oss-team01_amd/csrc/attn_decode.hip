@@ -20,6 +20,7 @@
 //     the T positions of a prompt are T such rows, which is all the prompt-pass attention is; two
 //     consecutive rows of a sequence then share a wave (8 heads each in the 16 operand columns).
 #include <algorithm>
+#include <mutex>
 #include <type_traits>
 
 #include "common.hpp"
@@ -544,6 +545,54 @@ extern "C" int gptoss_attn_decode(const float *q, const void *k_cache, const voi
                                   void *workspace, size_t workspace_bytes, void *stream) {
   return attn_launch(q, k_cache, v_cache, lens, sinks, out, B, 1, n_q, n_kv, head_dim, capacity, window,
                      max_len, workspace, workspace_bytes, stream);
+}
+
+// ---- the same call without a caller workspace ---------------------------------------------------
+// The chunk partials live in a device array that is part of the library image: every GPU the
+// library is loaded on holds its own copy until the process ends.  In host code the array's name
+// is only a handle; its device address is looked up once per device and kept.
+constexpr size_t ATTN_STATIC_SCRATCH_BYTES = (size_t)64 << 20;
+static __device__ __align__(256) unsigned char scratch[ATTN_STATIC_SCRATCH_BYTES];
+
+constexpr int ATTN_MAX_DEVICES = 64;
+static std::mutex g_scratch_mutex;
+static void *g_scratch_ptr[ATTN_MAX_DEVICES];  // per device, nullptr until looked up there
+
+// address of the calling thread's current device's copy of `scratch`
+static int static_scratch(void **ptr) {
+  int dev = -1;
+  GPTOSS_HIP(hipGetDevice(&dev));
+  GPTOSS_REQUIRE(dev >= 0 && dev < ATTN_MAX_DEVICES, GPTOSS_ERR_STATE,
+                 "attn_decode_static: device ordinal %d outside 0..%d", dev, ATTN_MAX_DEVICES - 1);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void *p = nullptr;
+    GPTOSS_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    GPTOSS_REQUIRE(p && aligned(p, 256), GPTOSS_ERR_HIP, "attn_decode_static: no address for the scratch array");
+    g_scratch_ptr[dev] = p;
+  }
+  *ptr = g_scratch_ptr[dev];
+  return GPTOSS_OK;
+}
+
+extern "C" size_t gptoss_attn_decode_static_max_bytes(void) { return ATTN_STATIC_SCRATCH_BYTES; }
+
+extern "C" int gptoss_attn_decode_static(const float *q, const void *k_cache, const void *v_cache,
+                                         const int *lens, const float *sinks, void *out, int B, int n_q,
+                                         int n_kv, int head_dim, int capacity, int window, int max_len,
+                                         void *stream) {
+  const size_t need = gptoss_attn_workspace_bytes(B, n_q, n_kv, head_dim, max_len);
+  GPTOSS_REQUIRE(need > 0, GPTOSS_ERR_DIM, "attn_decode_static: non-positive dimension");
+  GPTOSS_REQUIRE(need <= ATTN_STATIC_SCRATCH_BYTES, GPTOSS_ERR_WORKSPACE,
+                 "attn_decode_static: B=%d n_q=%d head_dim=%d max_len=%d needs %zu bytes of chunk partials, the "
+                 "built-in scratch holds %zu; use gptoss_attn_decode with a workspace", B, n_q, head_dim,
+                 max_len, need, ATTN_STATIC_SCRATCH_BYTES);
+  void *ptr = nullptr;
+  int rc = static_scratch(&ptr);
+  if (rc != GPTOSS_OK) return rc;
+  // every partial a merge reads was written by this call's first kernel: nothing to clear
+  return attn_launch(q, k_cache, v_cache, lens, sinks, out, B, 1, n_q, n_kv, head_dim, capacity, window,
+                     max_len, ptr, ATTN_STATIC_SCRATCH_BYTES, stream);
 }
 
 __global__ __launch_bounds__(256) void prefill_lens_kernel(int *lens, int rows, int T, int pos0) {

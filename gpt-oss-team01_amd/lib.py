@@ -75,6 +75,8 @@ SIGNATURES = {
     "gptoss_attn_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),
     "gptoss_attn_decode": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _sz,
                                 _vp]),
+    "gptoss_attn_decode_static_max_bytes": (_sz, []),
+    "gptoss_attn_decode_static": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "gptoss_engine_create": (_i, [C.POINTER(Config), _vp, _i, _i, _i, C.c_uint64,
                                   C.POINTER(_vp)]),
     "gptoss_engine_step": (_i, [_vp, _vp, _i, _i, _vp]),

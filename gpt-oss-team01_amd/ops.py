@@ -178,6 +178,21 @@ class AttnDecode:
         return out
 
 
+def attn_decode_static(q, cache: KVCache, lens, n_q, sinks=None, window=0, max_len=None, out=None):
+    """gptoss_attn_decode_static: the decode attention on the library's built-in scratch (no workspace,
+    no allocation inside the call; `out` is the caller's)."""
+    _need_gpu()
+    L = _l.load()
+    B = q.shape[0]
+    assert q.dtype == torch.float32 and q.is_contiguous() and lens.dtype == torch.int32
+    if out is None:
+        out = torch.empty(B, n_q, cache.D, dtype=torch.bfloat16, device=q.device)
+    _l.check(L.gptoss_attn_decode_static(_ptr(q), _ptr(cache.k), _ptr(cache.v), _ptr(lens), _ptr(sinks),
+                                         _ptr(out), B, n_q, cache.n_kv, cache.D, cache.cap, window,
+                                         int(max_len), _stream()))
+    return out
+
+
 class AttnPrefill:
     """The decode attention for T consecutive positions of every sequence at once:
     q [B,T,n_q,D] fp32 -> out [B,T,n_q,D] bf16; row (b,t) sees cached positions <= pos0 + t."""

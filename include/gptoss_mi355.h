@@ -185,6 +185,21 @@ int gptoss_attn_decode(const float *q, const void *k_cache, const void *v_cache,
                        int capacity, int window, int max_len, void *workspace,
                        size_t workspace_bytes, void *stream);
 
+/* gptoss_attn_decode for callers that cannot allocate or bring a workspace (code under HIP graph
+ * capture, serving loops and harnesses that forbid hipMalloc).  No counterpart in the reference.
+ * Same arguments, arithmetic and results as gptoss_attn_decode; the chunk partials of long
+ * sequences go to a device array built into the library (64 MiB, held by every GPU the library
+ * runs on until the process ends).  The call allocates nothing.  Refused with
+ * GPTOSS_ERR_WORKSPACE when gptoss_attn_workspace_bytes(B, n_q, n_kv, head_dim, max_len) exceeds
+ * gptoss_attn_decode_static_max_bytes() (e.g. 256 sequences x 64 heads x 64 up to 4096 positions
+ * need 39 MiB).  Nothing in the array has to start at zero.  All calls on one GPU share the array:
+ * calls that overlap on one GPU (two streams, two threads) race; calls on one stream do not.  The
+ * first call on a device looks the array's address up (make it outside a graph capture). */
+size_t gptoss_attn_decode_static_max_bytes(void);
+int gptoss_attn_decode_static(const float *q, const void *k_cache, const void *v_cache, const int *lens,
+                              const float *sinks, void *out, int B, int n_q, int n_kv, int head_dim,
+                              int capacity, int window, int max_len, void *stream);
+
 /* The same attention for T consecutive positions of every sequence at once (prompt processing):
  * q fp32 [B, T, n_q, D] and out bf16 [B, T, n_q, D]; row (b, t) attends to the cached positions up
  * to pos0 + t of sequence b, with the arithmetic gptoss_attn_decode uses for lens = pos0 + t + 1,
