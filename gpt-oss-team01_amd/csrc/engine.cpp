@@ -419,6 +419,13 @@ extern "C" int gptoss_engine_create(const gptoss_config *cfg, const float *host_
   GPTOSS_REQUIRE(max_batch >= 1 && max_seq >= 1 && max_seq <= c.seq_len, GPTOSS_ERR_DIM,
                  "engine_create: need max_batch >= 1 and 1 <= max_seq <= seq_len (%d)", c.seq_len);
   GPTOSS_REQUIRE(c.sliding_window >= 0, GPTOSS_ERR_DIM, "engine_create: negative sliding window");
+  // the GEMM kernels address their operands and results with 32-bit element offsets
+  {
+    const long long widest = std::max<long long>({qkv_dim, H, 2ll * I, (flags & (GPTOSS_ENGINE_LOGITS | GPTOSS_ENGINE_PRECISE)) ? V : 0});
+    GPTOSS_REQUIRE((long long)max_batch * widest < (1ll << 32), GPTOSS_ERR_DIM,
+                   "engine_create: max_batch x the widest activation row (%lld elements%s) must stay below 2^32 "
+                   "(max_batch=%d)", widest, widest == V ? ", the logits of GPTOSS_ENGINE_LOGITS" : "", max_batch);
+  }
 
   gptoss_engine *e = new gptoss_engine();
   e->cfg = c;

@@ -585,16 +585,25 @@ __global__ __launch_bounds__(GEMM_THREADS, (gemm_two_per_cu(MBMAX, FP4) ? 4 : 2)
   }
 }
 
+template <int MBMAX>
+constexpr size_t gemm_smem_bytes() {
+  return (size_t)3 * MBMAX * 32 * LDS_ROW * sizeof(bf16_t);
+}
+
+// The kernels use more dynamic LDS than a launch gets by default; the limit is raised for every
+// instantiation of a translation unit in one go (gemm_prepare_device in moe_gemm.hip, once per
+// device), not at an instantiation's first launch, so a first call may sit inside a graph capture
+// and concurrent first calls from several host threads do not race.
+template <int MBMAX, bool GATHER, int EPI, bool FP4>
+hipError_t gemm_set_attr() {
+  return hipFuncSetAttribute(reinterpret_cast<const void *>(grouped_gemm_kernel<MBMAX, GATHER, EPI, FP4>),
+                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)gemm_smem_bytes<MBMAX>());
+}
+
 template <int MBMAX, bool GATHER, int EPI, bool FP4>
 int launch_gemm(const GemmParams &p, int max_tiles, hipStream_t s) {
-  static bool attr_done = false;
-  size_t smem = (size_t)3 * MBMAX * 32 * LDS_ROW * sizeof(bf16_t);
+  const size_t smem = gemm_smem_bytes<MBMAX>();
   auto kern = grouped_gemm_kernel<MBMAX, GATHER, EPI, FP4>;
-  if (!attr_done) {
-    GPTOSS_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-    attr_done = true;
-  }
   int total = max_tiles * p.n_col_tiles;
   int grid = ((total + 7) / 8) * 8;
   // resident workgroups: one of 8 waves (2 per SIMD) per CU, or two where the registers allow
@@ -628,5 +637,21 @@ int launch_gemm(const GemmParams &p, int max_tiles, hipStream_t s) {
   template int launch_gemm<3, false, EPI_ARGMAX, FP4V>(const GemmParams &, int, hipStream_t);  \
   template int launch_gemm<4, false, EPI_ARGMAX, FP4V>(const GemmParams &, int, hipStream_t);  \
   template int launch_gemm<5, false, EPI_ARGMAX, FP4V>(const GemmParams &, int, hipStream_t);
+
+#define GPTOSS_GEMM_ATTR_ROW(M, FP4V)                                            \
+  if (err == hipSuccess) err = gemm_set_attr<M, true, EPI_SWIGLU, FP4V>();       \
+  if (err == hipSuccess) err = gemm_set_attr<M, false, EPI_F32, FP4V>();         \
+  if (err == hipSuccess) err = gemm_set_attr<M, false, EPI_ARGMAX, FP4V>();
+
+#define GPTOSS_GEMM_SET_ATTRS(NAME, FP4V) \
+  hipError_t NAME() {                     \
+    hipError_t err = hipSuccess;          \
+    GPTOSS_GEMM_ATTR_ROW(1, FP4V)         \
+    GPTOSS_GEMM_ATTR_ROW(2, FP4V)         \
+    GPTOSS_GEMM_ATTR_ROW(3, FP4V)         \
+    GPTOSS_GEMM_ATTR_ROW(4, FP4V)         \
+    GPTOSS_GEMM_ATTR_ROW(5, FP4V)         \
+    return err;                           \
+  }
 
 }  // namespace gptoss

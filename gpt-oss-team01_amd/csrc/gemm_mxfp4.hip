@@ -3,4 +3,5 @@
 
 namespace gptoss {
 GPTOSS_GEMM_INSTANTIATE(true)
+GPTOSS_GEMM_SET_ATTRS(gemm_set_attrs_mxfp4, true)
 }  // namespace gptoss

@@ -1,5 +1,7 @@
 // Host side of the grouped/dense GEMMs (kernel dispatch), the weighted combine kernel and the
 // weight repacking kernels.  The GEMM kernel itself is in gemm_kernel.hpp.
+#include <mutex>
+
 #include "common.hpp"
 #include "gemm.hpp"
 
@@ -211,8 +213,35 @@ static int dispatch_rows(const GemmParams &p, int rows_per_tile, int max_tiles, 
   return fail(GPTOSS_ERR_DIM, "run_gemm: unsupported rows_per_tile %d", rows_per_tile);
 }
 
+hipError_t gemm_set_attrs_bf16();   // gemm_bf16.hip
+hipError_t gemm_set_attrs_mxfp4();  // gemm_mxfp4.hip
+
+// Raises the dynamic-LDS limit of every GEMM kernel on the calling thread's current device, the
+// first time that device launches one.
+static int gemm_prepare_device() {
+  constexpr int MAX_DEV = 64;
+  static std::mutex mu;
+  static bool done[MAX_DEV];
+  int dev = 0;
+  GPTOSS_HIP(hipGetDevice(&dev));
+  GPTOSS_REQUIRE(dev >= 0 && dev < MAX_DEV, GPTOSS_ERR_STATE, "run_gemm: device ordinal %d outside 0..%d", dev, MAX_DEV - 1);
+  std::lock_guard<std::mutex> lock(mu);
+  if (!done[dev]) {
+    GPTOSS_HIP(gemm_set_attrs_bf16());
+    GPTOSS_HIP(gemm_set_attrs_mxfp4());
+    done[dev] = true;
+  }
+  return GPTOSS_OK;
+}
+
 int run_gemm(const GemmParams &p, bool gather, int epi, int rows_per_tile, int max_tiles,
              hipStream_t s) {
+  // output and operand offsets inside the kernels are 32-bit element counts
+  const long long max_rows = p.tiles ? (long long)max_tiles * rows_per_tile : p.dense_rows;
+  GPTOSS_REQUIRE(max_rows * p.N < (1ll << 32) && max_rows * p.K < (1ll << 32), GPTOSS_ERR_DIM,
+                 "run_gemm: rows x columns must stay below 2^32 elements (rows<=%lld N=%d K=%d)", max_rows, p.N, p.K);
+  int prc = gemm_prepare_device();
+  if (prc != GPTOSS_OK) return prc;
   if (gather && epi == EPI_SWIGLU) return dispatch_rows<true, EPI_SWIGLU>(p, rows_per_tile, max_tiles, s);
   if (!gather && epi == EPI_F32) return dispatch_rows<false, EPI_F32>(p, rows_per_tile, max_tiles, s);
   if (!gather && epi == EPI_ARGMAX && p.tiles == nullptr && p.amax_val && p.amax_idx)

@@ -128,4 +128,8 @@ def test_engine_entry_points_validate_before_touching_a_device(lib):
     cfg = lib.Config(4096, 256, 8, 4, 256, 4, 32, 8, 2, 64, 4096, 150000.0, 32.0, 128, 7.0)
     h = C.c_void_p()
     assert L.gptoss_engine_create(C.byref(cfg), p, 2, 16, lib.ENGINE_PRECISE | lib.ENGINE_SYNTHETIC, 0, C.byref(h)) == 6
+    # 32-bit element offsets inside the GEMM kernels: a logits buffer of 2^32 floats or more is refused
+    big = lib.Config(201088, 2880, 32, 4, 2880, 24, 64, 64, 8, 64, 4096, 150000.0, 32.0, 128, 7.0)
+    assert L.gptoss_engine_create(C.byref(big), None, 21400, 16, lib.ENGINE_SYNTHETIC | lib.ENGINE_LOGITS, 0, C.byref(h)) == 2
+    assert "2^32" in lib.last_error()
     assert L.gptoss_engine_create(C.byref(cfg), p, 2, 16, lib.ENGINE_PRECISE | lib.ENGINE_MXFP4_EXPERTS, 0, C.byref(h)) == 6
