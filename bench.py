@@ -381,6 +381,38 @@ def bench_e2e(ops, torch, n_req=1024, n_prompt=128, n_decode=256, scheduler=True
                       "window 128 on even layers; 1024 seqs x (128 prompt + 256 decoded)"}
 
 
+def bench_loader(ops, torch):
+    """Loader: an fp32 payload in .bin tensor order with the GPT-OSS-20B dimensions and two blocks
+    (11.2 GB in host memory) through gptoss_engine_create's pinned, double-buffered staging into the
+    kernels' bf16 layouts; GB/s of fp32 payload, second of two runs."""
+    import dataclasses
+    import numpy as np
+    synth = importlib.import_module("gpt-oss-team01_amd.synth")
+    binfmt = importlib.import_module("gpt-oss-team01_amd.binfmt")
+    cfg = dataclasses.replace(synth.gptoss20b_config(max_seq_len=64), n_layers=2)
+    flat = np.empty(binfmt.n_weight_floats(cfg), np.float32)
+    g = torch.Generator(device="cuda").manual_seed(5)
+    off = 0
+    for name, shape in binfmt.tensor_shapes(cfg).items():
+        n = int(np.prod(shape))
+        lead = shape[0] if len(shape) > 2 else 1
+        per = n // lead
+        for i in range(lead):
+            x = torch.randn(per, device="cuda", generator=g) * 0.02
+            flat[off + i * per: off + (i + 1) * per] = x.to(torch.bfloat16).float().cpu().numpy()
+        off += n
+    times = []
+    for _ in range(2):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        eng = ops.Engine(cfg, flat, max_batch=1, max_seq=16, prefill=False, keep_logits=False)
+        times.append(time.perf_counter() - t0)
+        eng.close()
+    return {"payload_gb": round(flat.nbytes / 1e9, 2), "seconds": round(times[-1], 3),
+            "gbs": round(flat.nbytes / times[-1] / 1e9, 1),
+            "what": "fp32 host payload (20B dimensions, 2 blocks) -> packed bf16 device weights, PCIe included"}
+
+
 def main():
     args = parse()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -426,6 +458,8 @@ def main():
     if not args.no_e2e:
         torch.cuda.empty_cache()
         extra["e2e_20b"] = bench_e2e(ops, torch, scheduler=not args.no_sched)
+        torch.cuda.empty_cache()
+        extra["loader"] = bench_loader(ops, torch)
 
     if cpu is not None and "e2e_20b" in extra:
         # whole-model CPU figure: not run (84 GB of fp32 weights, minutes per token); scaled from the

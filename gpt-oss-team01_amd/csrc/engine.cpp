@@ -8,6 +8,7 @@
 #include <string.h>
 
 #include <algorithm>
+#include <thread>
 #include <vector>
 
 #include "common.hpp"
@@ -88,12 +89,42 @@ struct gptoss_engine {
 
 namespace {
 
+// Host -> device staging of the fp32 payload: two pinned host buffers and two device buffers.
+// Chunk i is copied by the host into pinned[i % 2] (several threads), sent with an asynchronous
+// copy on its own stream, and converted/packed by a kernel on the engine's stream; the copy of chunk
+// i+1 and the host's work on chunk i+2 overlap that kernel.  Events order the reuse of either
+// buffer; the host only ever waits for the copy issued two chunks earlier.  Replaces the host-side
+// transposes and synchronous uploads of getp-csrc/src/alloc.cpp:27-35,112-127.
+struct Stager {
+  hipStream_t copy = nullptr;
+  float *pinned[2] = {nullptr, nullptr}, *dev[2] = {nullptr, nullptr};
+  hipEvent_t h2d_done[2] = {nullptr, nullptr}, consumed[2] = {nullptr, nullptr};
+  size_t elems = 0;   // floats per buffer
+  unsigned next = 0;
+};
+
+// plain copy by a few threads: one thread reaches a fraction of what the host memory can deliver
+static void host_copy(float *dst, const float *src, size_t n) {
+  constexpr int T = 6;
+  if (n < ((size_t)1 << 20)) {
+    memcpy(dst, src, n * sizeof(float));
+    return;
+  }
+  std::thread th[T - 1];
+  const size_t per = (n + T - 1) / T;
+  for (int i = 1; i < T; i++) {
+    const size_t lo = std::min(n, per * i), hi = std::min(n, per * (i + 1));
+    th[i - 1] = std::thread([=] { memcpy(dst + lo, src + lo, (hi - lo) * sizeof(float)); });
+  }
+  memcpy(dst, src, std::min(n, per) * sizeof(float));
+  for (int i = 1; i < T; i++) th[i - 1].join();
+}
+
 struct Builder {
   gptoss_engine *e;
   int rc = GPTOSS_OK;
-  // staging for the fp32 -> device layout conversion
-  float *stage_f32 = nullptr;
-  bf16_t *stage_bf16 = nullptr;
+  Stager st;                      // fp32 payload on its way to the device (host weights only)
+  bf16_t *stage_bf16 = nullptr;   // synthetic weights before packing
   size_t stage_elems = 0;
   // MXFP4 expert storage: unpacked codes and scales of one staging chunk, and the flag the
   // requantisation kernel raises when a value has no exact MXFP4 representation
@@ -121,12 +152,62 @@ struct Builder {
     if (rc == GPTOSS_OK && err != hipSuccess) rc = fail(GPTOSS_ERR_HIP, "engine: %s: %s", what, hipGetErrorString(err));
   }
 
+  void stager_create(size_t elems) {
+    st.elems = elems;
+    hip(hipStreamCreate(&st.copy), "hipStreamCreate");
+    for (int i = 0; i < 2 && ok(); i++) {
+      hip(hipHostMalloc((void **)&st.pinned[i], elems * sizeof(float), hipHostMallocDefault), "staging hipHostMalloc");
+      hip(hipMalloc((void **)&st.dev[i], elems * sizeof(float)), "staging hipMalloc");
+      hip(hipEventCreateWithFlags(&st.h2d_done[i], hipEventDisableTiming), "hipEventCreate");
+      hip(hipEventCreateWithFlags(&st.consumed[i], hipEventDisableTiming), "hipEventCreate");
+    }
+  }
+  void stager_destroy() {
+    if (st.copy) (void)hipStreamSynchronize(st.copy);
+    for (int i = 0; i < 2; i++) {
+      if (st.pinned[i]) (void)hipHostFree(st.pinned[i]);
+      if (st.dev[i]) (void)hipFree(st.dev[i]);
+      if (st.h2d_done[i]) (void)hipEventDestroy(st.h2d_done[i]);
+      if (st.consumed[i]) (void)hipEventDestroy(st.consumed[i]);
+    }
+    if (st.copy) (void)hipStreamDestroy(st.copy);
+    st = Stager();
+  }
+  // n floats of the payload -> a device buffer the engine's stream may read once this returns (the
+  // wait is enqueued, not performed); release(slot) after the kernels that read it are enqueued
+  const float *stage_in(const float *host, size_t n, int *slot) {
+    const int sl = (int)(st.next++ & 1);
+    *slot = sl;
+    if (!ok()) return nullptr;
+    // pinned[sl] is free once the copy that last read it has finished (an event never recorded is complete)
+    hip(hipEventSynchronize(st.h2d_done[sl]), "hipEventSynchronize");
+    if (!ok()) return nullptr;
+    host_copy(st.pinned[sl], host, n);
+    // dev[sl] is free once the kernels that last read it have finished
+    hip(hipStreamWaitEvent(st.copy, st.consumed[sl], 0), "hipStreamWaitEvent");
+    hip(hipMemcpyAsync(st.dev[sl], st.pinned[sl], n * sizeof(float), hipMemcpyHostToDevice, st.copy), "H2D");
+    hip(hipEventRecord(st.h2d_done[sl], st.copy), "hipEventRecord");
+    hip(hipStreamWaitEvent(e->stream, st.h2d_done[sl], 0), "hipStreamWaitEvent");
+    return st.dev[sl];
+  }
+  void release(int slot) { hip(hipEventRecord(st.consumed[slot], e->stream), "hipEventRecord"); }
+
   // fp32 host tensor -> fp32 device tensor
   float *upload_f32(const float *host, size_t n, uint64_t seed, float mean, float std) {
     float *d = alloc<float>(n);
     if (!ok()) return nullptr;
-    if (host) hip(hipMemcpyAsync(d, host, n * sizeof(float), hipMemcpyHostToDevice, e->stream), "H2D");
-    else check(run_synth_f32(d, n, seed, mean, std, e->stream));
+    if (!host) {
+      check(run_synth_f32(d, n, seed, mean, std, e->stream));
+      return d;
+    }
+    for (size_t o = 0; o < n && ok(); o += st.elems) {
+      const size_t c = std::min(st.elems, n - o);
+      int slot;
+      const float *src = stage_in(host + o, c, &slot);
+      if (!ok()) break;
+      hip(hipMemcpyAsync(d + o, src, c * sizeof(float), hipMemcpyDeviceToDevice, e->stream), "D2D");
+      release(slot);
+    }
     return d;
   }
 
@@ -136,34 +217,28 @@ struct Builder {
     size_t per = (size_t)n_out * n_in;
     bf16_t *dst = alloc<bf16_t>(per * n_mat);
     if (!ok()) return nullptr;
-    int group = (int)std::max<size_t>(1, stage_elems / per);
     if (per > stage_elems) {
       rc = fail(GPTOSS_ERR_DIM, "engine: a %d x %d matrix exceeds the staging buffer", n_out, n_in);
       return nullptr;
     }
+    int group = (int)std::max<size_t>(1, stage_elems / per);
     for (int m0 = 0; m0 < n_mat && ok(); m0 += group) {
       int nm = std::min(group, n_mat - m0);
       size_t n = per * nm;
-      const void *src;
-      int flags = pack_flags;
       if (host) {
-        hip(hipMemcpyAsync(stage_f32, host + per * m0, n * sizeof(float), hipMemcpyHostToDevice, e->stream), "H2D");
-        src = stage_f32;
-        flags |= GPTOSS_PACK_SRC_FP32;
+        int slot;
+        const float *src = stage_in(host + per * m0, n, &slot);
+        if (!ok()) break;
+        if (pack) check(gptoss_pack_weight(src, dst + per * m0, nm, n_out, n_in, pack_flags | GPTOSS_PACK_SRC_FP32, e->stream));
+        else check(run_f32_to_bf16(src, dst + per * m0, n, e->stream));
+        release(slot);
       } else {
+        // one stream, in order: the staging buffer is rewritten only after the kernel that read it
         check(run_synth_bf16(stage_bf16, n, seed + 7919ull * (uint64_t)m0, 0.f, std, e->stream));
-        src = stage_bf16;
+        if (!ok()) break;
+        if (pack) check(gptoss_pack_weight(stage_bf16, dst + per * m0, nm, n_out, n_in, pack_flags, e->stream));
+        else hip(hipMemcpyAsync(dst + per * m0, stage_bf16, n * sizeof(bf16_t), hipMemcpyDeviceToDevice, e->stream), "D2D");
       }
-      if (!ok()) break;
-      if (pack) {
-        check(gptoss_pack_weight(src, dst + per * m0, nm, n_out, n_in, flags, e->stream));
-      } else if (host) {
-        check(run_f32_to_bf16(stage_f32, dst + per * m0, n, e->stream));
-      } else {
-        hip(hipMemcpyAsync(dst + per * m0, stage_bf16, n * sizeof(bf16_t), hipMemcpyDeviceToDevice, e->stream), "D2D");
-      }
-      // the staging buffer is reused by the next group
-      hip(hipStreamSynchronize(e->stream), "sync");
     }
     return dst;
   }
@@ -184,15 +259,17 @@ struct Builder {
       const int nm = std::min(group, n_mat - m0);
       const size_t n_blocks = per * nm / 32;
       if (host) {
-        hip(hipMemcpyAsync(stage_f32, host + per * m0, per * nm * sizeof(float), hipMemcpyHostToDevice, e->stream), "H2D");
-        check(run_requant_mxfp4(stage_f32, n_blocks, q_blocks, q_scales, q_not_exact, e->stream));
+        int slot;
+        const float *src = stage_in(host + per * m0, per * nm, &slot);
+        if (!ok()) break;
+        check(run_requant_mxfp4(src, n_blocks, q_blocks, q_scales, q_not_exact, e->stream));
+        release(slot);
       } else {
         // scale exponents -13..-5: weights of the order of 0.02, as the bf16 synthetic weights
         check(run_synth_mxfp4(q_blocks, q_scales, n_blocks, seed + 7919ull * (uint64_t)m0, -5, e->stream));
       }
       if (!ok()) break;
       check(gptoss_pack_mxfp4(q_blocks, q_scales, dst + mat_bytes * m0, nm, n_out, n_in, pack_flags, e->stream));
-      hip(hipStreamSynchronize(e->stream), "sync");
     }
     return reinterpret_cast<bf16_t *>(dst);
   }
@@ -455,8 +532,8 @@ extern "C" int gptoss_engine_create(const gptoss_config *cfg, const float *host_
   // staging: large enough for one expert's gate/up matrix, one qkv matrix and a slice of the
   // (un)embedding table
   size_t biggest = std::max({(size_t)2 * I * H, (size_t)qkv_dim * H, (size_t)H * nq * D, (size_t)E * H});
-  b.stage_elems = std::max<size_t>(biggest, (size_t)16 << 20);
-  if (!synthetic) b.hip(hipMalloc((void **)&b.stage_f32, b.stage_elems * sizeof(float)), "staging hipMalloc");
+  b.stage_elems = std::max<size_t>(biggest, (size_t)32 << 20);
+  if (!synthetic) b.stager_create(b.stage_elems);
   else b.hip(hipMalloc((void **)&b.stage_bf16, b.stage_elems * sizeof(bf16_t)), "staging hipMalloc");
   const bool mxfp4 = (flags & GPTOSS_ENGINE_MXFP4_EXPERTS) != 0;
   if (mxfp4) {
@@ -491,25 +568,20 @@ extern "C" int gptoss_engine_create(const gptoss_config *cfg, const float *host_
       for (int r0 = 0; r0 < V && b.ok(); r0 += rows_per) {
         int nr = std::min(rows_per, V - r0);
         size_t n = (size_t)nr * H;
-        const void *s;
-        int fl = 0;
         if (src) {
-          b.hip(hipMemcpyAsync(b.stage_f32, src + (size_t)r0 * H, n * sizeof(float), hipMemcpyHostToDevice, e->stream), "H2D");
-          s = b.stage_f32;
-          fl = GPTOSS_PACK_SRC_FP32;
+          int slot;
+          const float *sp = b.stage_in(src + (size_t)r0 * H, n, &slot);
+          if (!b.ok()) break;
+          // fragment order is blocked by 32 output rows, so a slice of rows packs independently
+          if (pass == 0) b.check(run_f32_to_bf16(sp, dst + (size_t)r0 * H, n, e->stream));
+          else b.check(gptoss_pack_weight(sp, dst + (size_t)r0 * H, 1, nr, H, GPTOSS_PACK_SRC_FP32, e->stream));
+          b.release(slot);
         } else {
           b.check(run_synth_bf16(b.stage_bf16, n, next_seed(), 0.f, STD, e->stream));
-          s = b.stage_bf16;
+          if (!b.ok()) break;
+          if (pass == 0) b.hip(hipMemcpyAsync(dst + (size_t)r0 * H, b.stage_bf16, n * sizeof(bf16_t), hipMemcpyDeviceToDevice, e->stream), "D2D");
+          else b.check(gptoss_pack_weight(b.stage_bf16, dst + (size_t)r0 * H, 1, nr, H, 0, e->stream));
         }
-        if (!b.ok()) break;
-        if (pass == 0) {
-          if (src) b.check(run_f32_to_bf16(b.stage_f32, dst + (size_t)r0 * H, n, e->stream));
-          else b.hip(hipMemcpyAsync(dst + (size_t)r0 * H, b.stage_bf16, n * sizeof(bf16_t), hipMemcpyDeviceToDevice, e->stream), "D2D");
-        } else {
-          // fragment order is blocked by 32 output rows, so a slice of rows packs independently
-          b.check(gptoss_pack_weight(s, dst + (size_t)r0 * H, 1, nr, H, fl, e->stream));
-        }
-        b.hip(hipStreamSynchronize(e->stream), "sync");
       }
     }
   }
@@ -563,7 +635,9 @@ extern "C" int gptoss_engine_create(const gptoss_config *cfg, const float *host_
       b.rc = fail(GPTOSS_ERR_STATE, "engine_create: GPTOSS_ENGINE_MXFP4_EXPERTS needs expert weights that are exactly "
                                     "representable in MXFP4 (e2m1 codes, one power-of-two scale per 32 inputs)");
   }
-  if (b.stage_f32) (void)hipFree(b.stage_f32);
+  // the staging buffers are freed below: everything that reads them must have finished
+  b.hip(hipStreamSynchronize(e->stream), "sync");
+  b.stager_destroy();
   if (b.stage_bf16) (void)hipFree(b.stage_bf16);
   if (b.q_blocks) (void)hipFree(b.q_blocks);
   if (b.q_scales) (void)hipFree(b.q_scales);
@@ -1040,6 +1114,44 @@ extern "C" int gptoss_engine_generate(gptoss_engine *e, const int *host_prompts,
                                       long long *n_generated) {
   return gptoss_engine_generate_ragged(e, host_prompts, host_n_prompt, prompt_stride, n_req, max_seq_len, nullptr,
                                        host_out, n_generated);
+}
+
+// Device view of one weight tensor in the layout the kernels read.
+extern "C" int gptoss_engine_tensor_view(gptoss_engine *e, int tensor, int layer, void **ptr, size_t *bytes) {
+  GPTOSS_REQUIRE(e && ptr && bytes, GPTOSS_ERR_NULL, "engine_tensor_view: null pointer");
+  GPTOSS_REQUIRE(!(e->flags & GPTOSS_ENGINE_PRECISE), GPTOSS_ERR_STATE,
+                 "engine_tensor_view: GPTOSS_ENGINE_PRECISE keeps the fp32 payload as it is");
+  const gptoss_config &c = e->cfg;
+  const size_t H = c.hidden_dim, V = c.vocab_size, E = c.n_experts, I = c.intermediate_dim;
+  const size_t nq = c.n_attn_heads, nkv = c.n_kv_heads, D = c.head_dim, qkv_dim = (nq + 2 * nkv) * D;
+  const bool per_layer = tensor >= GPTOSS_TENSOR_ATTN_NORM;
+  GPTOSS_REQUIRE(tensor >= 0 && tensor <= GPTOSS_TENSOR_B2, GPTOSS_ERR_DIM, "engine_tensor_view: unknown tensor %d", tensor);
+  GPTOSS_REQUIRE(!per_layer || (layer >= 0 && layer < c.n_layers), GPTOSS_ERR_DIM,
+                 "engine_tensor_view: layer %d outside 0..%d", layer, c.n_layers - 1);
+  const bool q4 = (e->flags & GPTOSS_ENGINE_MXFP4_EXPERTS) != 0;
+  auto expert_bytes = [&](size_t n_out, size_t n_in) {
+    return q4 ? gptoss_packed_mxfp4_bytes((int)E, (int)n_out, (int)n_in) : E * n_out * n_in * sizeof(bf16_t);
+  };
+  const LayerWeights *w = per_layer ? &e->layers[layer] : nullptr;
+  switch (tensor) {
+    case GPTOSS_TENSOR_EMBEDDING: *ptr = e->embedding; *bytes = V * H * 2; break;
+    case GPTOSS_TENSOR_UNEMBEDDING: *ptr = e->unembedding; *bytes = V * H * 2; break;
+    case GPTOSS_TENSOR_FINAL_NORM: *ptr = e->final_norm; *bytes = H * 4; break;
+    case GPTOSS_TENSOR_ATTN_NORM: *ptr = w->attn_norm; *bytes = H * 4; break;
+    case GPTOSS_TENSOR_MLP_NORM: *ptr = w->mlp_norm; *bytes = H * 4; break;
+    case GPTOSS_TENSOR_W_QKV: *ptr = w->w_qkv; *bytes = qkv_dim * H * 2; break;
+    case GPTOSS_TENSOR_B_QKV: *ptr = w->b_qkv; *bytes = qkv_dim * 4; break;
+    case GPTOSS_TENSOR_W_O: *ptr = w->w_o; *bytes = H * nq * D * 2; break;
+    case GPTOSS_TENSOR_B_O: *ptr = w->b_o; *bytes = H * 4; break;
+    case GPTOSS_TENSOR_SINKS: *ptr = w->sinks; *bytes = nq * 4; break;
+    case GPTOSS_TENSOR_W_ROUTER: *ptr = w->w_router; *bytes = E * H * 2; break;
+    case GPTOSS_TENSOR_B_ROUTER: *ptr = w->b_router; *bytes = E * 4; break;
+    case GPTOSS_TENSOR_W1: *ptr = w->w1; *bytes = expert_bytes(2 * I, H); break;
+    case GPTOSS_TENSOR_B1: *ptr = w->b1; *bytes = E * 2 * I * 4; break;
+    case GPTOSS_TENSOR_W2: *ptr = w->w2; *bytes = expert_bytes(H, I); break;
+    default: *ptr = w->b2; *bytes = E * H * 4; break;
+  }
+  return GPTOSS_OK;
 }
 
 // Device views for tests and tracing: logits of the last step [B,V] and the residual stream.

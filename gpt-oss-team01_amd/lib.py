@@ -24,6 +24,12 @@ ENGINE_NO_PREFILL = 8
 ENGINE_MXFP4_EXPERTS = 16
 
 
+#: GPTOSS_TENSOR_* of gptoss_engine_tensor_view, in the header's order
+TENSORS = ("embedding", "unembedding", "final_norm", "attn_norm", "mlp_norm", "qkv_weight", "qkv_bias",
+           "out_weight", "out_bias", "sinks", "gate_weight", "gate_bias", "mlp1_weight", "mlp1_bias",
+           "mlp2_weight", "mlp2_bias")
+
+
 class GptossError(RuntimeError):
     def __init__(self, code, msg):
         super().__init__(f"{ERR_NAMES.get(code, code)}: {msg}")
@@ -87,6 +93,7 @@ SIGNATURES = {
     "gptoss_attn_prefill": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _sz, _vp]),
     "gptoss_engine_generate": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp, C.POINTER(C.c_longlong)]),
     "gptoss_engine_destroy": (None, [_vp]),
+    "gptoss_engine_tensor_view": (_i, [_vp, _i, _i, C.POINTER(_vp), C.POINTER(_sz)]),
     "gptoss_engine_debug_views": (_i, [_vp, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_sz)]),
 }
 

@@ -348,6 +348,19 @@ class Engine:
             raise RuntimeError(f"hipMemcpy failed: {rc}")
         return host.numpy()
 
+    def tensor(self, name, layer=0):
+        """Copy of one weight tensor as the engine holds it on the device (uint8, flat);
+        `name` is the tensor's name in binfmt.tensor_shapes."""
+        p, n = C.c_void_p(), C.c_size_t()
+        _l.check(self.L.gptoss_engine_tensor_view(self._h, _l.TENSORS.index(name), int(layer),
+                                                  C.byref(p), C.byref(n)))
+        out = torch.empty(n.value, dtype=torch.uint8, device="cuda")
+        torch.cuda.synchronize()
+        rc = C.CDLL("libamdhip64.so").hipMemcpy(C.c_void_p(out.data_ptr()), p, C.c_size_t(n.value), 3)
+        if rc != 0:
+            raise RuntimeError(f"hipMemcpy failed: {rc}")
+        return out
+
     def device_bytes(self):
         nb = C.c_size_t()
         _l.check(self.L.gptoss_engine_debug_views(self._h, None, None, C.byref(nb)))

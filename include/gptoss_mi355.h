@@ -306,6 +306,20 @@ void gptoss_engine_destroy(gptoss_engine *e);
  * the last step, and the bytes of device memory the engine holds.  Outputs may be NULL. */
 int gptoss_engine_debug_views(gptoss_engine *e, float **logits, float **x, size_t *device_bytes);
 
+/* Device view of one weight tensor as the engine holds it after loading: the counterpart of the
+ * fields of the reference's OurTransformerWeights (getp-csrc/include/config.hpp:50-158), which its
+ * loader fills tensor by tensor (getp-csrc/src/alloc.cpp:6-197).  Matrices are bf16: embedding and
+ * router row-major, every other matrix in gptoss_pack_weight order (mlp1 with GPTOSS_PACK_GLU),
+ * expert matrices in gptoss_pack_mxfp4 order under GPTOSS_ENGINE_MXFP4_EXPERTS; vectors are fp32.
+ * `layer` is ignored for the three tensors the model has once. */
+enum {
+  GPTOSS_TENSOR_EMBEDDING = 0, GPTOSS_TENSOR_UNEMBEDDING, GPTOSS_TENSOR_FINAL_NORM,
+  GPTOSS_TENSOR_ATTN_NORM, GPTOSS_TENSOR_MLP_NORM, GPTOSS_TENSOR_W_QKV, GPTOSS_TENSOR_B_QKV,
+  GPTOSS_TENSOR_W_O, GPTOSS_TENSOR_B_O, GPTOSS_TENSOR_SINKS, GPTOSS_TENSOR_W_ROUTER,
+  GPTOSS_TENSOR_B_ROUTER, GPTOSS_TENSOR_W1, GPTOSS_TENSOR_B1, GPTOSS_TENSOR_W2, GPTOSS_TENSOR_B2
+};
+int gptoss_engine_tensor_view(gptoss_engine *e, int tensor, int layer, void **ptr, size_t *bytes);
+
 #ifdef __cplusplus
 }
 #endif
