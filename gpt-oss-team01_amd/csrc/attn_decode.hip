@@ -12,10 +12,17 @@
 //   * K is stored [sequence, kv head, slot, d]: a wave reads 16 slots x 128 B = 2 KB contiguous
 //     per 128-bit load pair; V is stored in 32-slot blocks already in V^T operand order, 1 KB
 //     contiguous per load; position p lives in slot p % capacity (ring buffer for window layers);
-//   * long contexts are cut into chunks (flash-decoding): partial (max, sum, O) per chunk, merged
-//     with the sink by a small second kernel; sequences that fit one chunk finish in the first.
-//     The chunk length is a constant, so a row's result is the same whatever else is in the
-//     launch;
+//   * contexts of up to ATT_CHUNK slots are one wave's single pass;
+//   * longer contexts, few sequences: cut into chunks (flash-decoding), one wave each: partial
+//     (max, sum, O) per chunk go to the workspace and a small second kernel merges them with the
+//     sink.  The chunk length is a constant, so a row's result is the same whatever else is in
+//     the launch;
+//   * longer contexts, many sequences (enough to fill the chip with one workgroup per sequence
+//     and kv head): the four waves of a workgroup share one (sequence, kv head), wave w taking the
+//     64-slot blocks w, w+4, ..., and merge their states with the sink in LDS.  Nothing but the
+//     result is written: 20 MB of partials written next to a saturated K/V read stream cost
+//     38 us of a 260 us launch (256 sequences of 512..4096 positions), their merge kernel 11 more.
+//     Workgroups are dealt longest sequence first;
 //   * several query rows may share one sequence's cache (rows_per_seq), each with its own length:
 //     the T positions of a prompt are T such rows, which is all the prompt-pass attention is; two
 //     consecutive rows of a sequence then share a wave (8 heads each in the 16 operand columns).
@@ -42,6 +49,10 @@ struct AttnParams {
   int B, n_q, n_kv, G, cap, window, max_chunks, max_len;
   int rows_per_seq;    // query rows per cached sequence: row b reads the cache of sequence b / rows_per_seq
   float scale_log2e;   // log2(e) / sqrt(D)
+  int only_single;     // chunked kernels: leave rows of more than one chunk to the workgroup-per-row kernel
+  const int2 *order;   // workgroup-per-row kernel: (row, its length) by descending slot span (nullptr: row order)
+  int2 *order_out;     // chunked kernels: when set, one extra workgroup (the last) writes that order
+  int order_buckets;   // slot-span buckets (of 64 slots) the order distinguishes
 };
 
 struct SeqRange {
@@ -75,19 +86,83 @@ __device__ __forceinline__ SeqRange seq_range(int len, int cap, int window, int 
   return r;
 }
 
+// Rows by descending slot span, rows of a single chunk last: the order in which the
+// workgroup-per-row kernel is dealt its rows, so that the longest start first and the launch ends
+// on the shortest.  A counting sort over spans in units of 64 slots by one workgroup of 256
+// threads; rows of equal span come in any order (the order only schedules, no result depends on
+// it).  Each entry carries the row's length, which saves the consumer a dependent load.
+constexpr int ATT_ORDER_BUCKETS = 2048;
+
+__device__ __forceinline__ void attn_write_order(const AttnParams &p, int *hist /* [2*(ATT_ORDER_BUCKETS+1)] */) {
+  const int tid = threadIdx.x;
+  const int nbk = min(p.order_buckets, ATT_ORDER_BUCKETS) + 1;
+  int *start = hist + ATT_ORDER_BUCKETS + 1;
+  for (int i = tid; i < nbk; i += 256) hist[i] = 0;
+  __syncthreads();
+  auto key_of = [&](int len) {
+    const SeqRange r = seq_range(len, p.cap, p.window, p.max_len);
+    return r.nchunks > 1 ? min(nbk - 1, (r.s_end - r.s_begin + ATT_BLOCK - 1) / ATT_BLOCK) : 0;
+  };
+  for (int b = tid; b < p.B; b += 256) atomicAdd(&hist[key_of(p.lens[b])], 1);
+  __syncthreads();
+  // start[k] = number of rows with a larger key; thread t owns `per` consecutive buckets from the top
+  const int per = (nbk + 255) / 256;
+  int local = 0;
+  for (int i = 0; i < per; i++) {
+    const int k = nbk - 1 - (tid * per + i);
+    if (k >= 0) local += hist[k];
+  }
+  __shared__ int scan[256];
+  scan[tid] = local;
+  __syncthreads();
+  for (int off = 1; off < 256; off <<= 1) {
+    const int v = (tid >= off) ? scan[tid - off] : 0;
+    __syncthreads();
+    scan[tid] += v;
+    __syncthreads();
+  }
+  int run = scan[tid] - local;   // rows in the buckets above this thread's
+  for (int i = 0; i < per; i++) {
+    const int k = nbk - 1 - (tid * per + i);
+    if (k >= 0) {
+      start[k] = run;
+      run += hist[k];
+    }
+  }
+  __syncthreads();
+  for (int b = tid; b < p.B; b += 256) {
+    const int len = p.lens[b];
+    const int pos = atomicAdd(&start[key_of(len)], 1);
+    p.order_out[pos] = make_int2(b, len);
+  }
+}
+
 // PAIR (prompt passes, at most 8 query heads per kv head, ring not wrapped): a wave serves two
 // consecutive query rows of one sequence, row b in operand columns 0-7 and row b+1 in columns 8-15,
 // from one pass over the K/V blocks either of them needs.  Columns are independent in both MFMAs
 // and a block outside a row's own range is a no-op for its columns (scores -inf: max unchanged,
 // rescale factor exactly 1, probabilities exactly 0), so each row's result equals that of the
 // one-row kernel bit for bit.
-template <int D, bool PAIR>
+//
+// WG (many sequences, contexts of more than one chunk): the workgroup's four waves serve one
+// (row, kv head); wave w walks the 64-slot blocks w, w+4, ... of the row's slot range and the four
+// states are merged in LDS.
+template <int D, bool PAIR, bool WG = false>
 __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
+  static_assert(!(PAIR && WG), "a workgroup per row serves one row");
   constexpr int KS = D / 32;   // k-steps of the score MFMA
   constexpr int DB = D / 16;   // 16-row blocks of O^T
+  constexpr int STRIDE = WG ? 4 * ATT_BLOCK : ATT_BLOCK;   // slots between two blocks of one wave
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int item = blockIdx.x * 4 + wave;  // wave-uniform: everything derived from it stays scalar
+  if constexpr (!WG) {
+    if (p.order_out && blockIdx.x == gridDim.x - 1) {   // the extra workgroup of a launch that precedes the rows kernel
+      __shared__ int order_lds[2 * (ATT_ORDER_BUCKETS + 1)];
+      attn_write_order(p, order_lds);
+      return;
+    }
+  }
+  const int item = WG ? blockIdx.x : blockIdx.x * 4 + wave;  // wave-uniform: everything derived from it stays scalar
   const int g = item % p.n_kv;
   const int rest = item / p.n_kv;
   // work units per kv head and chunk: rows, or pairs of rows formed inside each sequence
@@ -96,16 +171,28 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
   const int units = PAIR ? (p.B / p.rows_per_seq) * pairs_per_seq : p.B;
   const int unit = rest % units;
   const int pair_seq = unit / pairs_per_seq, pair_idx = unit - pair_seq * pairs_per_seq;
-  const int b = PAIR ? pair_seq * p.rows_per_seq + 2 * pair_idx : unit;
+  int2 ordered = make_int2(unit, 0);
+  if (WG && p.order) {
+    ordered = p.order[unit];
+    ordered.x = __builtin_amdgcn_readfirstlane(ordered.x);
+    ordered.y = __builtin_amdgcn_readfirstlane(ordered.y);
+  }
+  const int b = PAIR ? pair_seq * p.rows_per_seq + 2 * pair_idx : ordered.x;
   // late chunks first: only long sequences have them, so the sparse part of the grid runs while
   // the chip is still filling and the grid ends on chunk 0, which every sequence has
-  const int chunk_id = p.max_chunks - 1 - rest / units;
+  const int chunk_id = WG ? 0 : p.max_chunks - 1 - rest / units;
   if (chunk_id < 0) return;
-  const SeqRange r = seq_range(__builtin_amdgcn_readfirstlane(p.lens[b]), p.cap, p.window, p.max_len);
+  SeqRange r = seq_range((WG && p.order) ? ordered.y : __builtin_amdgcn_readfirstlane(p.lens[b]), p.cap, p.window,
+                         p.max_len);
+  if (WG) {
+    if (r.nchunks <= 1) return;   // the whole workgroup: such rows belong to the one-wave kernel
+    r.chunk = r.s_end - r.s_begin;  // the workgroup walks the whole range
+  }
   // the second row of a pair: the next row of the same sequence, when there is one
   const bool two = PAIR && 2 * pair_idx + 1 < p.rows_per_seq;
   const SeqRange r1 = two ? seq_range(__builtin_amdgcn_readfirstlane(p.lens[b + 1]), p.cap, p.window, p.max_len) : r;
-  const bool act0 = chunk_id < r.nchunks, act1 = two && chunk_id < r1.nchunks;
+  const bool act0 = WG || (chunk_id < r.nchunks && !(p.only_single && r.nchunks > 1));
+  const bool act1 = two && chunk_id < r1.nchunks && !(p.only_single && r1.nchunks > 1);
   if (!act0 && !act1) return;
   // position held by slot s is s + pos_base, or cap less when that would lie beyond the last one
   const int pos_base = (r.len > 0) ? ((r.len - 1) / p.cap) * p.cap : 0;
@@ -118,7 +205,7 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
   const int c0_0 = r.s_begin + chunk_id * r.chunk, c0_1 = r1.s_begin + chunk_id * r1.chunk;
   const int hi0 = act0 ? min(r.s_end, c0_0 + r.chunk) : 0, hi1 = act1 ? min(r1.s_end, c0_1 + r1.chunk) : 0;
   const int lo0 = max(c0_0, r.t_lo), lo1 = max(c0_1, r1.t_lo);
-  const int c0 = !PAIR ? c0_0 : (act0 && act1) ? min(c0_0, c0_1) : act0 ? c0_0 : c0_1;
+  const int c0 = WG ? c0_0 + wave * ATT_BLOCK : !PAIR ? c0_0 : (act0 && act1) ? min(c0_0, c0_1) : act0 ? c0_0 : c0_1;
   const int c1 = !PAIR ? hi0 : max(hi0, hi1);
   const int n = lane & 15, c = lane >> 4;
   const int G = p.G;
@@ -289,22 +376,64 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
   };
 
   if (c1 > c0) {
+    // Every call of step() knows how many loads were requested after the block it consumes: one
+    // block's worth in the steady state, none for the last block.  (With the request under a
+    // condition of its own the wait counts have to assume it was skipped, and every block waits for
+    // the one just requested.)
     int blk = c0;
     while (true) {
-      if (blk + ATT_BLOCK < c1) load_kv(blk + ATT_BLOCK, R1{});  // wave-uniform: no reload of the last block
+      if (blk + STRIDE >= c1) { step(blk, R0{}); break; }
+      load_kv(blk + STRIDE, R1{});
       step(blk, R0{});
-      blk += ATT_BLOCK;
-      if (blk >= c1) break;
-      if (blk + ATT_BLOCK < c1) load_kv(blk + ATT_BLOCK, R0{});
+      blk += STRIDE;
+      if (blk + STRIDE >= c1) { step(blk, R1{}); break; }
+      load_kv(blk + STRIDE, R0{});
       step(blk, R1{});
-      blk += ATT_BLOCK;
-      if (blk >= c1) break;
+      blk += STRIDE;
     }
   }
 
   // ---- per-head totals: sum the partial denominators of the 4 lanes that share a head --------
   l_run += __shfl_xor(l_run, 16, 64);
   l_run += __shfl_xor(l_run, 32, 64);
+  if constexpr (WG) {
+    // the four waves' states (a wave without a block holds the neutral one: max -1e30, sum 0, O 0)
+    // meet in LDS and are merged with the sink in wave order, by the formula of attn_reduce_kernel
+    __shared__ float lds_o[4 * 16 * D];
+    __shared__ float lds_ml[4 * 16 * 2];
+    if (col_live) {
+#pragma unroll
+      for (int db = 0; db < DB; db++)
+        *reinterpret_cast<f32x4 *>(&lds_o[(wave * 16 + n) * D + db * 16 + c * 4]) = o[db];
+      if (c == 0) {
+        lds_ml[(wave * 16 + n) * 2] = m_run;
+        lds_ml[(wave * 16 + n) * 2 + 1] = l_run;
+      }
+    }
+    __syncthreads();
+    constexpr int TPP = D / 4;  // threads per head
+    const int hm = threadIdx.x / TPP, d4 = (threadIdx.x % TPP) * 4;
+    if (hm >= G) return;
+    const int hq = g * G + hm;
+    const float sink2 = p.sinks ? p.sinks[hq] * 1.4426950408889634f : -INFINITY;
+    float M = sink2;
+#pragma unroll
+    for (int w = 0; w < 4; w++) M = fmaxf(M, lds_ml[(w * 16 + hm) * 2]);
+    float denom = exp2f(sink2 - M);
+    f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int w = 0; w < 4; w++) {
+      const float wgt = exp2f(lds_ml[(w * 16 + hm) * 2] - M);
+      denom += lds_ml[(w * 16 + hm) * 2 + 1] * wgt;
+      const f32x4 ow = *reinterpret_cast<const f32x4 *>(&lds_o[(w * 16 + hm) * D + d4]);
+#pragma unroll
+      for (int q = 0; q < 4; q++) acc[q] += ow[q] * wgt;
+    }
+    u32x2 pk = u32x2{pack_bf16x2(denom > 0.f ? acc[0] / denom : 0.f, denom > 0.f ? acc[1] / denom : 0.f),
+                     pack_bf16x2(denom > 0.f ? acc[2] / denom : 0.f, denom > 0.f ? acc[3] / denom : 0.f)};
+    *reinterpret_cast<u32x2 *>(p.out + ((size_t)b * p.n_q + hq) * D + d4) = pk;
+    return;
+  }
   if (!col_live) return;
   if (PAIR && !(second ? act1 : act0)) return;  // this row has no such chunk
   const int hq = g * G + hn;
@@ -415,18 +544,27 @@ __global__ __launch_bounds__(256) void kv_cache_write_kernel(bf16_t *__restrict_
 
 struct AttnPlan {
   int max_chunks;
-  size_t part_o_bytes, part_ml_bytes;
+  bool wide;          // many sequences: rows of more than one chunk get a workgroup each, no partials
+  size_t order_bytes, part_o_bytes, part_ml_bytes;
 };
 
-static AttnPlan attn_plan(int B, int n_q, int D, int max_len) {
+// Enough sequences that one workgroup per (sequence, kv head) fills the chip twice over: then long
+// rows are served by the workgroup-per-row kernel.  A property of the launch shape alone, so a
+// row's arithmetic depends on the number of sequences in the call but never on their contents.
+static bool attn_wide(int n_seq, int n_kv) { return (long long)n_seq * n_kv >= 512; }
+
+static AttnPlan attn_plan(int B, int rows_per_seq, int n_q, int n_kv, int D, int span) {
   AttnPlan pl;
   // most work items any row can have: a slot range can start up to 63 slots before the first
   // active position
-  const int longest = max_len + ATT_BLOCK - 1;
+  const int longest = span + ATT_BLOCK - 1;
   pl.max_chunks = (longest + ATT_CHUNK - 1) / ATT_CHUNK;
   if (pl.max_chunks < 1) pl.max_chunks = 1;
-  pl.part_o_bytes = align_up((size_t)B * pl.max_chunks * n_q * D * sizeof(float), 256);
-  pl.part_ml_bytes = align_up((size_t)B * pl.max_chunks * n_q * 2 * sizeof(float), 256);
+  pl.wide = pl.max_chunks > 1 && attn_wide(B / std::max(1, rows_per_seq), n_kv);
+  pl.order_bytes = align_up((size_t)B * sizeof(int2), 256);
+  const int stored_chunks = pl.wide ? 0 : pl.max_chunks;
+  pl.part_o_bytes = align_up((size_t)B * stored_chunks * n_q * D * sizeof(float), 256);
+  pl.part_ml_bytes = align_up((size_t)B * stored_chunks * n_q * 2 * sizeof(float), 256);
   return pl;
 }
 
@@ -460,10 +598,11 @@ extern "C" int gptoss_kv_cache_write(void *k_cache, void *v_cache, const void *k
 
 extern "C" size_t gptoss_attn_workspace_bytes(int B, int n_q, int n_kv, int head_dim, int max_len) {
   if (B <= 0 || n_q <= 0 || n_kv <= 0 || head_dim <= 0 || max_len <= 0) return 0;
-  // sized for a split into 256-slot work items, twice as fine as the kernel's: any window/capacity
-  // combination fits
-  int max_chunks = (max_len + ATT_BLOCK - 1 + 255) / 256;
-  return align_up((size_t)B * max_chunks * n_q * head_dim * sizeof(float), 256) +
+  // the row order of the workgroup-per-row kernel, or the chunk partials of the chunked one: sized
+  // for the larger of the two whatever window/capacity the call then has
+  int max_chunks = (max_len + ATT_BLOCK - 1 + ATT_CHUNK - 1) / ATT_CHUNK;
+  return align_up((size_t)B * sizeof(int2), 256) +
+         align_up((size_t)B * max_chunks * n_q * head_dim * sizeof(float), 256) +
          align_up((size_t)B * max_chunks * n_q * 2 * sizeof(float), 256);
 }
 
@@ -487,11 +626,10 @@ static int attn_launch(const float *q, const void *k_cache, const void *v_cache,
   // longest slot range one sequence can visit: the whole ring once it may have wrapped
   int span = (max_len > capacity) ? capacity
                                   : ((window > 0 && window < max_len) ? window : max_len);
-  AttnPlan pl = attn_plan(B, n_q, head_dim, span);
-  GPTOSS_REQUIRE(workspace && aligned(workspace, 256) &&
-                     workspace_bytes >= pl.part_o_bytes + pl.part_ml_bytes,
-                 GPTOSS_ERR_WORKSPACE, "attn_decode: workspace missing, misaligned or smaller than %zu bytes",
-                 pl.part_o_bytes + pl.part_ml_bytes);
+  AttnPlan pl = attn_plan(B, rows_per_seq, n_q, n_kv, head_dim, span);
+  const size_t need = pl.order_bytes + pl.part_o_bytes + pl.part_ml_bytes;
+  GPTOSS_REQUIRE(workspace && aligned(workspace, 256) && workspace_bytes >= need, GPTOSS_ERR_WORKSPACE,
+                 "attn_decode: workspace missing, misaligned or smaller than %zu bytes", need);
   AttnParams p;
   p.q = q;
   p.kc = (const bf16_t *)k_cache;
@@ -499,8 +637,9 @@ static int attn_launch(const float *q, const void *k_cache, const void *v_cache,
   p.lens = lens;
   p.sinks = sinks;
   p.out = (bf16_t *)out;
-  p.part_o = (float *)workspace;
-  p.part_ml = (float *)((unsigned char *)workspace + pl.part_o_bytes);
+  int2 *order = (int2 *)workspace;
+  p.part_o = (float *)((unsigned char *)workspace + pl.order_bytes);
+  p.part_ml = (float *)((unsigned char *)workspace + pl.order_bytes + pl.part_o_bytes);
   p.B = B;
   p.rows_per_seq = rows_per_seq;
   p.n_q = n_q;
@@ -508,15 +647,19 @@ static int attn_launch(const float *q, const void *k_cache, const void *v_cache,
   p.G = n_q / n_kv;
   p.cap = capacity;
   p.window = window;
-  p.max_chunks = pl.max_chunks;
+  p.max_chunks = pl.wide ? 1 : pl.max_chunks;
   p.max_len = max_len;
   p.scale_log2e = 1.4426950408889634f / sqrtf((float)head_dim);
+  p.only_single = pl.wide ? 1 : 0;
+  p.order = nullptr;
+  p.order_out = pl.wide ? order : nullptr;
+  p.order_buckets = (span + 2 * ATT_BLOCK - 1) / ATT_BLOCK;
   hipStream_t s = (hipStream_t)stream;
   // prompt passes put two consecutive rows of a sequence into one wave when the 16 operand columns
   // hold both rows' query heads and no ring can have wrapped (slot == position)
   const bool pair = rows_per_seq > 1 && B % rows_per_seq == 0 && p.G <= 8 && max_len <= capacity;
-  long long items = (long long)(pair ? (B / rows_per_seq) * ((rows_per_seq + 1) / 2) : B) * n_kv * pl.max_chunks;
-  int grid = (int)((items + 3) / 4);
+  long long items = (long long)(pair ? (B / rows_per_seq) * ((rows_per_seq + 1) / 2) : B) * n_kv * p.max_chunks;
+  int grid = (int)((items + 3) / 4) + (pl.wide ? 1 : 0);
   {
     TraceScope ts("attn_decode", s);
     if (head_dim == 64) {
@@ -528,7 +671,17 @@ static int attn_launch(const float *q, const void *k_cache, const void *v_cache,
     }
   }
   GPTOSS_LAUNCH_CHECK("attn_decode_kernel");
-  if (pl.max_chunks > 1) {
+  if (pl.wide) {
+    // rows of more than one chunk: a workgroup each, longest first (the order was written by the
+    // extra workgroup of the launch above)
+    p.order = order;
+    p.order_out = nullptr;
+    TraceScope ts("attn_decode_rows", s);
+    const int wgrid = B * n_kv;
+    if (head_dim == 64) attn_decode_kernel<64, false, true><<<wgrid, 256, 0, s>>>(p);
+    else attn_decode_kernel<32, false, true><<<wgrid, 256, 0, s>>>(p);
+    GPTOSS_LAUNCH_CHECK("attn_decode_kernel (workgroup per row)");
+  } else if (pl.max_chunks > 1) {
     int per_block = 256 / (head_dim / 4);
     int rgrid = (B * n_q + per_block - 1) / per_block;
     TraceScope ts("attn_reduce", s);
