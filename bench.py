@@ -222,8 +222,7 @@ def bench_attn(ops, torch, steps, warmup):
     caches = []
     for _ in range(2):
         c = ops.KVCache(B, n_kv, D, S)
-        c.k.normal_()
-        c.v.normal_()
+        c.kv.normal_()
         caches.append(c)
     q = torch.randn(B, n_q, D, device="cuda")
     sinks = torch.randn(n_q, device="cuda")

@@ -9,9 +9,10 @@
 //         S^T[token, head] = K[token, :] . Q^T[:, head]        (v_mfma_f32_16x16x32_bf16)
 //         O^T[d, head]    += V^T[d, token] . P^T[token, head]
 //     q and p are split into bf16 hi+lo parts (two MFMAs each) so they keep ~16 mantissa bits;
-//   * K is stored [sequence, kv head, slot, d]: a wave reads 16 slots x 128 B = 2 KB contiguous
-//     per 128-bit load pair; V is stored in 32-slot blocks already in V^T operand order, 1 KB
-//     contiguous per load; position p lives in slot p % capacity (ring buffer for window layers);
+//   * K and V of a (sequence, kv head) share one stream of 64-slot blocks (K rows of the block,
+//     then its V in V^T operand order, common.hpp): a wave reads 16 KB contiguous per block with
+//     128-bit loads, the four waves of a workgroup 64 KB; position p lives in slot p % capacity
+//     (ring buffer for window layers);
 //   * contexts of up to ATT_CHUNK slots are one wave's single pass;
 //   * longer contexts, few sequences: cut into chunks (flash-decoding), one wave each: partial
 //     (max, sum, O) per chunk go to the workspace and a small second kernel merges them with the
@@ -39,8 +40,7 @@ constexpr float NEG_BIG = -1.0e30f;
 
 struct AttnParams {
   const float *q;      // [B, n_q, D]
-  const bf16_t *kc;    // [B, n_kv, cap, D]
-  const bf16_t *vc;    // [B, n_kv, cap/32, D/16, 64, 8]
+  const bf16_t *kv;    // [B, n_kv, cap/64] blocks of K [64, D] + V [2, D/16, 64, 8]
   const int *lens;     // [B]
   const float *sinks;  // [n_q] or nullptr
   bf16_t *out;         // [B, n_q, D]
@@ -219,26 +219,26 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
   const float sink_logit = p.sinks ? p.sinks[head] : -INFINITY;
 
   const int seq = (p.rows_per_seq > 1) ? b / p.rows_per_seq : b;
-  const bf16_t *kbase = p.kc + ((size_t)(seq * p.n_kv + g) * p.cap) * D;
-  const bf16_t *vbase = p.vc + ((size_t)(seq * p.n_kv + g) * p.cap) * D;
-  // lane's K bytes for slot block `blk`: slot blk + tb*16 + n, d chunk c*KS*8 .. +KS*8
+  const bf16_t *plane = p.kv + kv_block_off(seq, g, p.n_kv, p.cap, D, 0);
+  // lane's K bytes of a block: slot tb*16 + n, d chunk c*KS*8 .. +KS*8; its V bytes: 8 elements per
+  // operand fragment
   const size_t k_lane = (size_t)n * D + c * KS * 8;
-  const size_t v_lane = (size_t)lane * 8;
+  const size_t v_lane = (size_t)KV_BLOCK * D + (size_t)lane * 8;
 
   u32x4 kreg[2][4][KS], vreg[2][2][DB];
   auto load_kv = [&](int blk, auto buf) {
     constexpr int R = decltype(buf)::value;
+    const bf16_t *bb = plane + (size_t)(blk >> 6) * (2 * KV_BLOCK * D);   // blk is a multiple of 64
 #pragma unroll
     for (int tb = 0; tb < 4; tb++)
 #pragma unroll
       for (int s = 0; s < KS; s++)
-        kreg[R][tb][s] = *reinterpret_cast<const u32x4 *>(kbase + (size_t)(blk + tb * 16) * D + k_lane + s * 8);
+        kreg[R][tb][s] = *reinterpret_cast<const u32x4 *>(bb + (size_t)(tb * 16) * D + k_lane + s * 8);
 #pragma unroll
     for (int grp = 0; grp < 2; grp++)
 #pragma unroll
       for (int db = 0; db < DB; db++)
-        vreg[R][grp][db] = *reinterpret_cast<const u32x4 *>(
-            vbase + ((size_t)((blk >> 5) + grp) * DB + db) * 512 + v_lane);
+        vreg[R][grp][db] = *reinterpret_cast<const u32x4 *>(bb + (size_t)(grp * DB + db) * 512 + v_lane);
   };
 
   // the first K/V block is requested before anything waits on q, so the cache stream of a work
@@ -518,8 +518,8 @@ __global__ __launch_bounds__(256) void attn_reduce_kernel(AttnParams p) {
   *reinterpret_cast<u32x2 *>(p.out + ((size_t)b * p.n_q + hq) * D + d4) = pk;
 }
 
-// Bulk cache write: rows [B, n_tok, n_kv, D] -> K [B, n_kv, cap, D], V in 32-slot operand blocks.
-__global__ __launch_bounds__(256) void kv_cache_write_kernel(bf16_t *__restrict__ kc, bf16_t *__restrict__ vc,
+// Bulk cache write: rows [B, n_tok, n_kv, D] -> the block layout of common.hpp.
+__global__ __launch_bounds__(256) void kv_cache_write_kernel(bf16_t *__restrict__ kv,
                                                              const bf16_t *__restrict__ k_rows,
                                                              const bf16_t *__restrict__ v_rows, int B,
                                                              int n_kv, int D, int cap, int pos0,
@@ -533,12 +533,9 @@ __global__ __launch_bounds__(256) void kv_cache_write_kernel(bf16_t *__restrict_
     int t = (int)(r % n_tok);
     int b = (int)(r / n_tok);
     int slot = (pos0 + t) % cap;
-    size_t base = ((size_t)(b * n_kv + g) * cap) * D;
-    kc[base + (size_t)slot * D + d] = k_rows[i];
-    int tt = slot & 31, within = tt & 15;
-    int lane = (within >> 2) * 16 + (d & 15);
-    int j = (tt >> 4) * 4 + (within & 3);
-    vc[base + ((size_t)(slot >> 5) * (D / 16) + (d >> 4)) * 512 + lane * 8 + j] = v_rows[i];
+    const size_t base = kv_block_off(b, g, n_kv, cap, D, slot);
+    kv[base + kv_k_elem(slot, d, D)] = k_rows[i];
+    kv[base + kv_v_elem(slot, d, D)] = v_rows[i];
   }
 }
 
@@ -573,14 +570,13 @@ static AttnPlan attn_plan(int B, int rows_per_seq, int n_q, int n_kv, int D, int
 using namespace gptoss;
 
 extern "C" size_t gptoss_kv_cache_bytes(int B, int n_kv, int head_dim, int capacity) {
-  if (B <= 0 || n_kv <= 0 || head_dim <= 0 || capacity <= 0) return 0;
-  return (size_t)B * n_kv * capacity * head_dim * sizeof(bf16_t);
+  if (B <= 0 || n_kv <= 0 || head_dim <= 0 || capacity <= 0 || capacity % KV_BLOCK) return 0;
+  return (size_t)B * n_kv * kv_plane_elems(capacity, head_dim) * sizeof(bf16_t);
 }
 
-extern "C" int gptoss_kv_cache_write(void *k_cache, void *v_cache, const void *k_rows,
-                                     const void *v_rows, int B, int n_kv, int head_dim,
-                                     int capacity, int pos0, int n_tok, void *stream) {
-  GPTOSS_REQUIRE(k_cache && v_cache && k_rows && v_rows, GPTOSS_ERR_NULL, "kv_cache_write: null pointer");
+extern "C" int gptoss_kv_cache_write(void *kv_cache, const void *k_rows, const void *v_rows, int B, int n_kv,
+                                     int head_dim, int capacity, int pos0, int n_tok, void *stream) {
+  GPTOSS_REQUIRE(kv_cache && k_rows && v_rows, GPTOSS_ERR_NULL, "kv_cache_write: null pointer");
   GPTOSS_REQUIRE(B > 0 && n_kv > 0 && (head_dim == 32 || head_dim == 64) && capacity > 0 &&
                      capacity % 64 == 0 && pos0 >= 0 && n_tok >= 0 && n_tok <= capacity,
                  GPTOSS_ERR_DIM,
@@ -589,9 +585,9 @@ extern "C" int gptoss_kv_cache_write(void *k_cache, void *v_cache, const void *k
   if (n_tok == 0) return GPTOSS_OK;
   size_t total = (size_t)B * n_tok * n_kv * head_dim;
   int grid = (int)((total + 255) / 256 > 65536 ? 65536 : (total + 255) / 256);
-  kv_cache_write_kernel<<<grid, 256, 0, (hipStream_t)stream>>>((bf16_t *)k_cache, (bf16_t *)v_cache,
-                                                               (const bf16_t *)k_rows, (const bf16_t *)v_rows,
-                                                               B, n_kv, head_dim, capacity, pos0, n_tok);
+  kv_cache_write_kernel<<<grid, 256, 0, (hipStream_t)stream>>>((bf16_t *)kv_cache, (const bf16_t *)k_rows,
+                                                               (const bf16_t *)v_rows, B, n_kv, head_dim, capacity,
+                                                               pos0, n_tok);
   GPTOSS_LAUNCH_CHECK("kv_cache_write_kernel");
   return GPTOSS_OK;
 }
@@ -607,11 +603,11 @@ extern "C" size_t gptoss_attn_workspace_bytes(int B, int n_q, int n_kv, int head
 }
 
 // B query rows; row b reads the cache of sequence b / rows_per_seq up to its own lens[b]
-static int attn_launch(const float *q, const void *k_cache, const void *v_cache, const int *lens,
+static int attn_launch(const float *q, const void *kv_cache, const int *lens,
                        const float *sinks, void *out, int B, int rows_per_seq, int n_q, int n_kv,
                        int head_dim, int capacity, int window, int max_len, void *workspace,
                        size_t workspace_bytes, void *stream) {
-  GPTOSS_REQUIRE(q && k_cache && v_cache && lens && out, GPTOSS_ERR_NULL, "attn_decode: null pointer");
+  GPTOSS_REQUIRE(q && kv_cache && lens && out, GPTOSS_ERR_NULL, "attn_decode: null pointer");
   GPTOSS_REQUIRE(B > 0 && n_q > 0 && n_kv > 0 && n_q % n_kv == 0 && n_q / n_kv <= 16, GPTOSS_ERR_DIM,
                  "attn_decode: need n_q %% n_kv == 0 and n_q/n_kv <= 16 (n_q=%d n_kv=%d)", n_q, n_kv);
   GPTOSS_REQUIRE(head_dim == 32 || head_dim == 64, GPTOSS_ERR_DIM,
@@ -621,7 +617,7 @@ static int attn_launch(const float *q, const void *k_cache, const void *v_cache,
   GPTOSS_REQUIRE(max_len <= capacity || (window > 0 && window <= capacity), GPTOSS_ERR_DIM,
                  "attn_decode: the cache must hold every active position (capacity=%d window=%d max_len=%d)",
                  capacity, window, max_len);
-  GPTOSS_REQUIRE(aligned(q, 16) && aligned(k_cache, 16) && aligned(v_cache, 16) && aligned(out, 8),
+  GPTOSS_REQUIRE(aligned(q, 16) && aligned(kv_cache, 16) && aligned(out, 8),
                  GPTOSS_ERR_ALIGN, "attn_decode: pointers must be 16-byte aligned");
   // longest slot range one sequence can visit: the whole ring once it may have wrapped
   int span = (max_len > capacity) ? capacity
@@ -632,8 +628,7 @@ static int attn_launch(const float *q, const void *k_cache, const void *v_cache,
                  "attn_decode: workspace missing, misaligned or smaller than %zu bytes", need);
   AttnParams p;
   p.q = q;
-  p.kc = (const bf16_t *)k_cache;
-  p.vc = (const bf16_t *)v_cache;
+  p.kv = (const bf16_t *)kv_cache;
   p.lens = lens;
   p.sinks = sinks;
   p.out = (bf16_t *)out;
@@ -692,11 +687,10 @@ static int attn_launch(const float *q, const void *k_cache, const void *v_cache,
   return GPTOSS_OK;
 }
 
-extern "C" int gptoss_attn_decode(const float *q, const void *k_cache, const void *v_cache,
-                                  const int *lens, const float *sinks, void *out, int B, int n_q,
-                                  int n_kv, int head_dim, int capacity, int window, int max_len,
-                                  void *workspace, size_t workspace_bytes, void *stream) {
-  return attn_launch(q, k_cache, v_cache, lens, sinks, out, B, 1, n_q, n_kv, head_dim, capacity, window,
+extern "C" int gptoss_attn_decode(const float *q, const void *kv_cache, const int *lens, const float *sinks,
+                                  void *out, int B, int n_q, int n_kv, int head_dim, int capacity, int window,
+                                  int max_len, void *workspace, size_t workspace_bytes, void *stream) {
+  return attn_launch(q, kv_cache, lens, sinks, out, B, 1, n_q, n_kv, head_dim, capacity, window,
                      max_len, workspace, workspace_bytes, stream);
 }
 
@@ -730,10 +724,9 @@ static int static_scratch(void **ptr) {
 
 extern "C" size_t gptoss_attn_decode_static_max_bytes(void) { return ATTN_STATIC_SCRATCH_BYTES; }
 
-extern "C" int gptoss_attn_decode_static(const float *q, const void *k_cache, const void *v_cache,
-                                         const int *lens, const float *sinks, void *out, int B, int n_q,
-                                         int n_kv, int head_dim, int capacity, int window, int max_len,
-                                         void *stream) {
+extern "C" int gptoss_attn_decode_static(const float *q, const void *kv_cache, const int *lens,
+                                         const float *sinks, void *out, int B, int n_q, int n_kv, int head_dim,
+                                         int capacity, int window, int max_len, void *stream) {
   const size_t need = gptoss_attn_workspace_bytes(B, n_q, n_kv, head_dim, max_len);
   GPTOSS_REQUIRE(need > 0, GPTOSS_ERR_DIM, "attn_decode_static: non-positive dimension");
   GPTOSS_REQUIRE(need <= ATTN_STATIC_SCRATCH_BYTES, GPTOSS_ERR_WORKSPACE,
@@ -744,8 +737,8 @@ extern "C" int gptoss_attn_decode_static(const float *q, const void *k_cache, co
   int rc = static_scratch(&ptr);
   if (rc != GPTOSS_OK) return rc;
   // every partial a merge reads was written by this call's first kernel: nothing to clear
-  return attn_launch(q, k_cache, v_cache, lens, sinks, out, B, 1, n_q, n_kv, head_dim, capacity, window,
-                     max_len, ptr, ATTN_STATIC_SCRATCH_BYTES, stream);
+  return attn_launch(q, kv_cache, lens, sinks, out, B, 1, n_q, n_kv, head_dim, capacity, window, max_len, ptr,
+                     ATTN_STATIC_SCRATCH_BYTES, stream);
 }
 
 __global__ __launch_bounds__(256) void prefill_lens_kernel(int *lens, int rows, int T, int pos0) {
@@ -761,8 +754,7 @@ extern "C" size_t gptoss_attn_prefill_workspace_bytes(int B, int T, int n_q, int
   return align_up(rows * sizeof(int), 256) + gptoss_attn_workspace_bytes((int)rows, n_q, n_kv, head_dim, max_len);
 }
 
-extern "C" int gptoss_attn_prefill(const float *q, const void *k_cache, const void *v_cache,
-                                   const float *sinks, void *out, int B, int T, int pos0, int n_q,
+extern "C" int gptoss_attn_prefill(const float *q, const void *kv_cache, const float *sinks, void *out, int B, int T, int pos0, int n_q,
                                    int n_kv, int head_dim, int capacity, int window, void *workspace,
                                    size_t workspace_bytes, void *stream) {
   GPTOSS_REQUIRE(B > 0 && T > 0 && pos0 >= 0 && (long long)B * T < (1ll << 24), GPTOSS_ERR_DIM,
@@ -777,6 +769,6 @@ extern "C" int gptoss_attn_prefill(const float *q, const void *k_cache, const vo
   int *lens = (int *)workspace;
   prefill_lens_kernel<<<(rows + 255) / 256, 256, 0, (hipStream_t)stream>>>(lens, rows, T, pos0);
   GPTOSS_LAUNCH_CHECK("prefill_lens_kernel");
-  return attn_launch(q, k_cache, v_cache, lens, sinks, out, rows, T, n_q, n_kv, head_dim, capacity, window,
+  return attn_launch(q, kv_cache, lens, sinks, out, rows, T, n_q, n_kv, head_dim, capacity, window,
                      pos0 + T, (unsigned char *)workspace + lens_bytes, workspace_bytes - lens_bytes, stream);
 }

@@ -62,7 +62,7 @@ const char *trace_name(int i) { return (i >= 0 && i < g_trace.count) ? g_trace.n
 }  // namespace gptoss
 
 extern "C" const char *gptoss_last_error_string(void) { return gptoss::last_error(); }
-extern "C" int gptoss_abi_version(void) { return 100; }
+extern "C" int gptoss_abi_version(void) { return 101; }
 extern "C" int gptoss_trace_set(void *const *start_events, void *const *stop_events, int n) {
   if (n < 0) return gptoss::fail(GPTOSS_ERR_DIM, "trace_set: negative count");
   return gptoss::trace_set(start_events, stop_events, n);

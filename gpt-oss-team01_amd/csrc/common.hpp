@@ -81,4 +81,24 @@ __device__ __forceinline__ bf16x8 as_bf16x8(u32x4 v) {
 
 __device__ __forceinline__ int lane_id() { return threadIdx.x & (WAVE - 1); }
 
+// ---- KV cache layout ---------------------------------------------------------------------------
+// One array per layer: for every (sequence, kv head) capacity/64 blocks of 64 slots; a block holds
+// the K rows of its slots, [64][D] bf16, followed by their V in the operand order of the second
+// attention MFMA, [2 groups of 32 slots][D/16][64 lanes][8].  A wave that walks a sequence reads
+// one contiguous 256*D-byte unit per 64 slots; position p lives in slot p % capacity.
+constexpr int KV_BLOCK = 64;
+__host__ __device__ __forceinline__ size_t kv_plane_elems(int cap, int D) { return (size_t)cap * D * 2; }
+// first element of the block that holds `slot` of (seq, g)
+__device__ __forceinline__ size_t kv_block_off(int seq, int g, int n_kv, int cap, int D, int slot) {
+  return ((size_t)(seq * n_kv + g) * (cap >> 6) + (slot >> 6)) * (size_t)(2 * KV_BLOCK * D);
+}
+// element offsets inside a block
+__device__ __forceinline__ int kv_k_elem(int slot, int d, int D) { return (slot & 63) * D + d; }
+__device__ __forceinline__ int kv_v_elem(int slot, int d, int D) {
+  const int tt = slot & 31, within = tt & 15;
+  const int lane = (within >> 2) * 16 + (d & 15);
+  const int j = (tt >> 4) * 4 + (within & 3);
+  return KV_BLOCK * D + (((slot & 63) >> 5) * (D >> 4) + (d >> 4)) * 512 + lane * 8 + j;
+}
+
 }  // namespace gptoss

@@ -35,7 +35,7 @@ struct LayerWeights {
   float *b1;
   bf16_t *w2;                     // packed [E][H,I]     (likewise)
   float *b2;
-  bf16_t *k_cache, *v_cache;
+  bf16_t *kv_cache;               // K and V of the layer, block layout of common.hpp
   int cache_cap;
   int window;                     // 0 = full attention
 };
@@ -71,7 +71,7 @@ struct gptoss_engine {
     int rows;  // 0: not available
     int *tokens;
     float *x, *qkv, *q, *tb2;
-    bf16_t *t, *attn_out, *k_scratch, *v_scratch;
+    bf16_t *t, *attn_out, *kv_scratch;
     size_t scratch_tokens;  // positions (summed over sequences) the scratch holds
     void *moe_ws, *attn_ws;
     size_t moe_ws_bytes, attn_ws_bytes;
@@ -620,13 +620,9 @@ extern "C" int gptoss_engine_create(const gptoss_config *cfg, const float *host_
     const bool windowed = W > 0 && (l % 2 == 0);
     w.window = windowed ? W : 0;
     w.cache_cap = windowed ? std::min(cap_full, (int)align_up((size_t)W, 64)) : cap_full;
-    size_t cache_elems = (size_t)max_batch * nkv * w.cache_cap * D;
-    w.k_cache = b.alloc<bf16_t>(cache_elems);
-    w.v_cache = b.alloc<bf16_t>(cache_elems);
-    if (b.ok()) {
-      b.hip(hipMemsetAsync(w.k_cache, 0, cache_elems * 2, e->stream), "memset");
-      b.hip(hipMemsetAsync(w.v_cache, 0, cache_elems * 2, e->stream), "memset");
-    }
+    size_t cache_elems = (size_t)max_batch * nkv * kv_plane_elems(w.cache_cap, D);
+    w.kv_cache = b.alloc<bf16_t>(cache_elems);
+    if (b.ok()) b.hip(hipMemsetAsync(w.kv_cache, 0, cache_elems * sizeof(bf16_t), e->stream), "memset");
   }
   if (mxfp4 && b.ok()) {
     int not_exact = 0;
@@ -693,16 +689,14 @@ extern "C" int gptoss_engine_create(const gptoss_config *cfg, const float *host_
     // rows of one launch: B sequences x T positions with B*T <= R and T <= max_seq
     pf.attn_ws_bytes = gptoss_attn_prefill_workspace_bytes(1, R, nq, nkv, D, std::min(R, max_seq));
     pf.attn_ws = b.alloc<unsigned char>(pf.attn_ws_bytes);
-    pf.k_scratch = pf.v_scratch = nullptr;
+    pf.kv_scratch = nullptr;
     pf.scratch_tokens = 0;
     if (W > 0 && max_seq > (int)align_up((size_t)W, 64)) {
       pf.scratch_tokens = (size_t)R + (size_t)64 * max_batch;
-      pf.k_scratch = b.alloc<bf16_t>(pf.scratch_tokens * nkv * D);
-      pf.v_scratch = b.alloc<bf16_t>(pf.scratch_tokens * nkv * D);
+      pf.kv_scratch = b.alloc<bf16_t>(pf.scratch_tokens * nkv * D * 2);
       // slots past a prompt's end are masked, but must hold finite values
       if (b.ok()) {
-        b.hip(hipMemsetAsync(pf.k_scratch, 0, pf.scratch_tokens * nkv * D * sizeof(bf16_t), e->stream), "memset");
-        b.hip(hipMemsetAsync(pf.v_scratch, 0, pf.scratch_tokens * nkv * D * sizeof(bf16_t), e->stream), "memset");
+        b.hip(hipMemsetAsync(pf.kv_scratch, 0, pf.scratch_tokens * nkv * D * 2 * sizeof(bf16_t), e->stream), "memset");
       }
     }
     if (b.ok()) pf.rows = R;
@@ -756,12 +750,12 @@ static int step_impl(gptoss_engine *e, const int *host_tokens, int pos, const in
     if (l == 0) STEP(run_rmsnorm(e->x, nullptr, w.attn_norm, e->t, nullptr, B, H, s));
     STEP(dense_gemm(e->t, w.w_qkv, w.b_qkv, e->qkv, EPI_F32, B, qkv_dim, H, s));
     if (host_pos)
-      STEP(run_rope_store_lens(e->qkv, e->q, w.k_cache, w.v_cache, e->cos_t, e->sin_t, B, nq, nkv, D,
+      STEP(run_rope_store_lens(e->qkv, e->q, w.kv_cache, e->cos_t, e->sin_t, B, nq, nkv, D,
                                w.cache_cap, e->d_lens, s));
     else
-      STEP(run_rope_store(e->qkv, e->q, w.k_cache, w.v_cache, e->cos_t, e->sin_t, B, nq, nkv, D,
+      STEP(run_rope_store(e->qkv, e->q, w.kv_cache, e->cos_t, e->sin_t, B, nq, nkv, D,
                           w.cache_cap, pos, s));
-    STEP(gptoss_attn_decode(e->q, w.k_cache, w.v_cache, e->d_lens, w.sinks, e->attn_out, B, nq, nkv, D,
+    STEP(gptoss_attn_decode(e->q, w.kv_cache, e->d_lens, w.sinks, e->attn_out, B, nq, nkv, D,
                             w.cache_cap, w.window, pos + 1, e->attn_ws, e->attn_ws_bytes, s));
     STEP(dense_gemm(e->attn_out, w.w_o, w.b_o, e->tb2, EPI_F32, B, H, nq * D, s));
     // x += attention branch, then the ffn norm (model.cpp:66)
@@ -850,21 +844,20 @@ static int prefill_chunk(gptoss_engine *e, const int *host_tokens, int seq0, int
     const LayerWeights &w = e->layers[l];
     if (l == 0) STEP(run_rmsnorm(pf.x, nullptr, w.attn_norm, pf.t, nullptr, rows, H, s));
     STEP(dense_gemm(pf.t, w.w_qkv, w.b_qkv, pf.qkv, EPI_F32, rows, qkv_dim, H, s));
-    const size_t seq_elems = (size_t)nkv * w.cache_cap * D;
-    bf16_t *kc = w.k_cache + seq_elems * seq0, *vc = w.v_cache + seq_elems * seq0;
+    bf16_t *kv = w.kv_cache + (size_t)nkv * kv_plane_elems(w.cache_cap, D) * seq0;
     if (T > w.cache_cap) {
       // a sliding-window ring shorter than the prompt: attention reads a linear copy of the
       // prompt's K/V, the ring receives the positions it would hold after T lock-step steps
       const int cap_t = (int)align_up((size_t)T, 64);
-      STEP(run_rope_store_rows(pf.qkv, pf.q, pf.k_scratch, pf.v_scratch, e->cos_t, e->sin_t, rows, T, nq, nkv, D,
+      STEP(run_rope_store_rows(pf.qkv, pf.q, pf.kv_scratch, e->cos_t, e->sin_t, rows, T, nq, nkv, D,
                                cap_t, 0, 0, s));
-      STEP(run_rope_store_rows(pf.qkv, nullptr, kc, vc, e->cos_t, e->sin_t, rows, T, nq, nkv, D, w.cache_cap, 0,
+      STEP(run_rope_store_rows(pf.qkv, nullptr, kv, e->cos_t, e->sin_t, rows, T, nq, nkv, D, w.cache_cap, 0,
                                T - w.cache_cap, s));
-      STEP(gptoss_attn_prefill(pf.q, pf.k_scratch, pf.v_scratch, w.sinks, pf.attn_out, Bc, T, 0, nq, nkv, D, cap_t,
+      STEP(gptoss_attn_prefill(pf.q, pf.kv_scratch, w.sinks, pf.attn_out, Bc, T, 0, nq, nkv, D, cap_t,
                                w.window, pf.attn_ws, pf.attn_ws_bytes, s));
     } else {
-      STEP(run_rope_store_rows(pf.qkv, pf.q, kc, vc, e->cos_t, e->sin_t, rows, T, nq, nkv, D, w.cache_cap, 0, 0, s));
-      STEP(gptoss_attn_prefill(pf.q, kc, vc, w.sinks, pf.attn_out, Bc, T, 0, nq, nkv, D, w.cache_cap, w.window,
+      STEP(run_rope_store_rows(pf.qkv, pf.q, kv, e->cos_t, e->sin_t, rows, T, nq, nkv, D, w.cache_cap, 0, 0, s));
+      STEP(gptoss_attn_prefill(pf.q, kv, w.sinks, pf.attn_out, Bc, T, 0, nq, nkv, D, w.cache_cap, w.window,
                                pf.attn_ws, pf.attn_ws_bytes, s));
     }
     STEP(dense_gemm(pf.attn_out, w.w_o, w.b_o, pf.tb2, EPI_F32, rows, H, nq * D, s));

@@ -108,7 +108,7 @@ __global__ __launch_bounds__(256) void rmsnorm_rows_kernel(float *__restrict__ x
 // reference: qkv_split_rope_store_kernel, layer_hip_batch.cpp:686-776
 __global__ __launch_bounds__(256) void rope_store_kernel(const float *__restrict__ qkv,
                                                          float *__restrict__ q_out,
-                                                         bf16_t *__restrict__ kc, bf16_t *__restrict__ vc,
+                                                         bf16_t *__restrict__ kv,
                                                          const float *__restrict__ cos_t,
                                                          const float *__restrict__ sin_t, int n_q,
                                                          int n_kv, int D, int cap, int pos0, int T,
@@ -148,18 +148,13 @@ __global__ __launch_bounds__(256) void rope_store_kernel(const float *__restrict
     const int g = p / quads, j4 = (p - g * quads) * 4;
     f32x4 lo, hi;
     rotate(row + q_dim + g * D, j4, lo, hi);
-    const size_t base = ((size_t)(b * n_kv + g) * cap + slot) * D;
-    *reinterpret_cast<u32x2 *>(kc + base + j4) = u32x2{pack_bf16x2(lo[0], lo[1]), pack_bf16x2(lo[2], lo[3])};
-    *reinterpret_cast<u32x2 *>(kc + base + half + j4) = u32x2{pack_bf16x2(hi[0], hi[1]), pack_bf16x2(hi[2], hi[3])};
+    bf16_t *krow = kv + kv_block_off(b, g, n_kv, cap, D, slot) + kv_k_elem(slot, 0, D);
+    *reinterpret_cast<u32x2 *>(krow + j4) = u32x2{pack_bf16x2(lo[0], lo[1]), pack_bf16x2(lo[2], lo[3])};
+    *reinterpret_cast<u32x2 *>(krow + half + j4) = u32x2{pack_bf16x2(hi[0], hi[1]), pack_bf16x2(hi[2], hi[3])};
   }
   for (int p = threadIdx.x; p < kv_dim; p += 256) {
     int g = p / D, d = p - g * D;
-    size_t base = ((size_t)(b * n_kv + g) * cap) * D;
-    int tt = slot & 31, within = tt & 15;
-    int lane = (within >> 2) * 16 + (d & 15);
-    int j = (tt >> 4) * 4 + (within & 3);
-    vc[base + ((size_t)(slot >> 5) * (D / 16) + (d >> 4)) * 512 + lane * 8 + j] =
-        f32_to_bf16(row[q_dim + kv_dim + p]);
+    kv[kv_block_off(b, g, n_kv, cap, D, slot) + kv_v_elem(slot, d, D)] = f32_to_bf16(row[q_dim + kv_dim + p]);
   }
 }
 
@@ -343,26 +338,26 @@ int run_gather_rows(const float *src, float *dst, int rows, int n, int stride, i
   return GPTOSS_OK;
 }
 
-int run_rope_store(const float *qkv, float *q_out, bf16_t *kc, bf16_t *vc, const float *cos_t,
+int run_rope_store(const float *qkv, float *q_out, bf16_t *kv, const float *cos_t,
                    const float *sin_t, int B, int n_q, int n_kv, int D, int cap, int pos,
                    hipStream_t s) {
-  return run_rope_store_rows(qkv, q_out, kc, vc, cos_t, sin_t, B, 1, n_q, n_kv, D, cap, pos, 0, s);
+  return run_rope_store_rows(qkv, q_out, kv, cos_t, sin_t, B, 1, n_q, n_kv, D, cap, pos, 0, s);
 }
 
-int run_rope_store_lens(const float *qkv, float *q_out, bf16_t *kc, bf16_t *vc, const float *cos_t,
+int run_rope_store_lens(const float *qkv, float *q_out, bf16_t *kv, const float *cos_t,
                         const float *sin_t, int B, int n_q, int n_kv, int D, int cap, const int *lens,
                         hipStream_t s) {
   TraceScope ts("rope_store", s);
-  rope_store_kernel<<<B, 256, 0, s>>>(qkv, q_out, kc, vc, cos_t, sin_t, n_q, n_kv, D, cap, 0, 1, 0, lens);
+  rope_store_kernel<<<B, 256, 0, s>>>(qkv, q_out, kv, cos_t, sin_t, n_q, n_kv, D, cap, 0, 1, 0, lens);
   GPTOSS_LAUNCH_CHECK("rope_store_kernel");
   return GPTOSS_OK;
 }
 
-int run_rope_store_rows(const float *qkv, float *q_out, bf16_t *kc, bf16_t *vc, const float *cos_t,
+int run_rope_store_rows(const float *qkv, float *q_out, bf16_t *kv, const float *cos_t,
                         const float *sin_t, int rows, int T, int n_q, int n_kv, int D, int cap, int pos0,
                         int store_from, hipStream_t s) {
   TraceScope ts("rope_store", s);
-  rope_store_kernel<<<rows, 256, 0, s>>>(qkv, q_out, kc, vc, cos_t, sin_t, n_q, n_kv, D, cap, pos0, T,
+  rope_store_kernel<<<rows, 256, 0, s>>>(qkv, q_out, kv, cos_t, sin_t, n_q, n_kv, D, cap, pos0, T,
                                          store_from, nullptr);
   GPTOSS_LAUNCH_CHECK("rope_store_kernel");
   return GPTOSS_OK;

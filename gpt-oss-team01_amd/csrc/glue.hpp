@@ -8,16 +8,16 @@ int run_embedding(const bf16_t *table, const int *tokens, float *x, int B, int H
 // x (+= residual) -> t_bf16 (and t_f32 when not null); residual may be null
 int run_rmsnorm(float *x, const float *residual, const float *weight, bf16_t *t_bf16, float *t_f32,
                 int B, int H, hipStream_t s);
-int run_rope_store(const float *qkv, float *q_out, bf16_t *kc, bf16_t *vc, const float *cos_t,
+int run_rope_store(const float *qkv, float *q_out, bf16_t *kv, const float *cos_t,
                    const float *sin_t, int B, int n_q, int n_kv, int D, int cap, int pos,
                    hipStream_t s);
 // rows = sequences * T: row r is position pos0 + r % T of sequence r / T; K/V of positions below
 // store_from are not stored; q_out may be null
-int run_rope_store_rows(const float *qkv, float *q_out, bf16_t *kc, bf16_t *vc, const float *cos_t,
+int run_rope_store_rows(const float *qkv, float *q_out, bf16_t *kv, const float *cos_t,
                         const float *sin_t, int rows, int T, int n_q, int n_kv, int D, int cap, int pos0,
                         int store_from, hipStream_t s);
 // one row per sequence, each at its own position lens[r] - 1
-int run_rope_store_lens(const float *qkv, float *q_out, bf16_t *kc, bf16_t *vc, const float *cos_t,
+int run_rope_store_lens(const float *qkv, float *q_out, bf16_t *kv, const float *cos_t,
                         const float *sin_t, int B, int n_q, int n_kv, int D, int cap, const int *lens,
                         hipStream_t s);
 // dst[i, :] = src[i * stride + offset, :]

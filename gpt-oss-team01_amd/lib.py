@@ -77,12 +77,11 @@ SIGNATURES = {
     "gptoss_pack_mxfp4": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "gptoss_moe_forward_mxfp4": (_i, [C.POINTER(MoeWeights), _vp, _i, _vp, _i, _vp, _sz, _vp]),
     "gptoss_kv_cache_bytes": (_sz, [_i, _i, _i, _i]),
-    "gptoss_kv_cache_write": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),
+    "gptoss_kv_cache_write": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),
     "gptoss_attn_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),
-    "gptoss_attn_decode": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _sz,
-                                _vp]),
+    "gptoss_attn_decode": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _sz, _vp]),
     "gptoss_attn_decode_static_max_bytes": (_sz, []),
-    "gptoss_attn_decode_static": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp]),
+    "gptoss_attn_decode_static": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "gptoss_engine_create": (_i, [C.POINTER(Config), _vp, _i, _i, _i, C.c_uint64,
                                   C.POINTER(_vp)]),
     "gptoss_engine_step": (_i, [_vp, _vp, _i, _i, _vp]),
@@ -90,7 +89,7 @@ SIGNATURES = {
     "gptoss_engine_step_ragged": (_i, [_vp, _vp, _vp, _i, _vp]),
     "gptoss_engine_generate_ragged": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp, _vp, C.POINTER(C.c_longlong)]),
     "gptoss_attn_prefill_workspace_bytes": (_sz, [_i, _i, _i, _i, _i, _i]),
-    "gptoss_attn_prefill": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _sz, _vp]),
+    "gptoss_attn_prefill": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _sz, _vp]),
     "gptoss_engine_generate": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp, C.POINTER(C.c_longlong)]),
     "gptoss_engine_destroy": (None, [_vp]),
     "gptoss_engine_tensor_view": (_i, [_vp, _i, _i, C.POINTER(_vp), C.POINTER(_sz)]),

@@ -142,8 +142,8 @@ class KVCache:
         if nbytes == 0 or capacity % 64:
             raise ValueError("KVCache: capacity must be a positive multiple of 64")
         alloc = torch.zeros if zero else torch.empty
-        self.k = alloc(nbytes // 2, dtype=torch.bfloat16, device=device)
-        self.v = alloc(nbytes // 2, dtype=torch.bfloat16, device=device)
+        #: K and V together, in the kernels' block layout
+        self.kv = alloc(nbytes // 2, dtype=torch.bfloat16, device=device)
 
     def write(self, k_rows, v_rows, pos0=0):
         """k_rows, v_rows: bf16 [B, n_tok, n_kv, D] for positions pos0 .. pos0+n_tok-1."""
@@ -151,9 +151,15 @@ class KVCache:
         assert (B, n_kv, D) == (self.B, self.n_kv, self.D)
         assert k_rows.dtype == torch.bfloat16 and v_rows.dtype == torch.bfloat16
         k_rows, v_rows = k_rows.contiguous(), v_rows.contiguous()
-        _l.check(self.L.gptoss_kv_cache_write(_ptr(self.k), _ptr(self.v), _ptr(k_rows),
-                                              _ptr(v_rows), B, n_kv, D, self.cap, pos0, n_tok,
-                                              _stream()))
+        _l.check(self.L.gptoss_kv_cache_write(_ptr(self.kv), _ptr(k_rows), _ptr(v_rows), B, n_kv, D,
+                                              self.cap, pos0, n_tok, _stream()))
+
+    def first(self, n_seq):
+        """A view of the first n_seq sequences (the layout is sequence-major)."""
+        c = KVCache.__new__(KVCache)
+        c.L, c.B, c.n_kv, c.D, c.cap = self.L, n_seq, self.n_kv, self.D, self.cap
+        c.kv = self.kv[: self.L.gptoss_kv_cache_bytes(n_seq, self.n_kv, self.D, self.cap) // 2]
+        return c
 
 
 class AttnDecode:
@@ -171,7 +177,7 @@ class AttnDecode:
         assert q.dtype == torch.float32 and q.is_contiguous() and lens.dtype == torch.int32
         if out is None:
             out = torch.empty(B, self.n_q, self.D, dtype=torch.bfloat16, device=q.device)
-        _l.check(self.L.gptoss_attn_decode(_ptr(q), _ptr(cache.k), _ptr(cache.v), _ptr(lens),
+        _l.check(self.L.gptoss_attn_decode(_ptr(q), _ptr(cache.kv), _ptr(lens),
                                            _ptr(sinks), _ptr(out), B, self.n_q, self.n_kv, self.D,
                                            cache.cap, window, max_len or self.max_len,
                                            _ptr(self.ws), self.ws_bytes, _stream()))
@@ -187,7 +193,7 @@ def attn_decode_static(q, cache: KVCache, lens, n_q, sinks=None, window=0, max_l
     assert q.dtype == torch.float32 and q.is_contiguous() and lens.dtype == torch.int32
     if out is None:
         out = torch.empty(B, n_q, cache.D, dtype=torch.bfloat16, device=q.device)
-    _l.check(L.gptoss_attn_decode_static(_ptr(q), _ptr(cache.k), _ptr(cache.v), _ptr(lens), _ptr(sinks),
+    _l.check(L.gptoss_attn_decode_static(_ptr(q), _ptr(cache.kv), _ptr(lens), _ptr(sinks),
                                          _ptr(out), B, n_q, cache.n_kv, cache.D, cache.cap, window,
                                          int(max_len), _stream()))
     return out
@@ -208,7 +214,7 @@ class AttnPrefill:
         B, T = q.shape[:2]
         assert q.dtype == torch.float32 and q.is_contiguous()
         out = torch.empty(B, T, self.n_q, self.D, dtype=torch.bfloat16, device=q.device)
-        _l.check(self.L.gptoss_attn_prefill(_ptr(q), _ptr(cache.k), _ptr(cache.v), _ptr(sinks), _ptr(out),
+        _l.check(self.L.gptoss_attn_prefill(_ptr(q), _ptr(cache.kv), _ptr(sinks), _ptr(out),
                                             B, T, pos0, self.n_q, self.n_kv, self.D, cache.cap, window,
                                             _ptr(self.ws), self.ws_bytes, _stream()))
         return out

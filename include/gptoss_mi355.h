@@ -157,19 +157,22 @@ int gptoss_moe_forward_mxfp4(const gptoss_moe_weights *w, const void *t, int B, 
 
 /* ------------------------------------------------------------------ decode attention ------- */
 
-/* The KV cache layout is internal (tiled for 128-bit streaming and MFMA operand order); size it
- * with gptoss_kv_cache_bytes and fill it with gptoss_kv_cache_write.  `capacity` = token slots per
+/* The KV cache of a layer is ONE array holding K and V (the reference keeps two tensors per layer,
+ * getp-csrc/src/alloc.cpp:239-262): per sequence and kv head, blocks of 64 token slots, each the
+ * K rows of its slots followed by their V in MFMA operand order, so that a wave streams one
+ * contiguous 16 KB unit per 64 slots.  The layout is internal: size the array with
+ * gptoss_kv_cache_bytes and fill it with gptoss_kv_cache_write.  `capacity` = token slots per
  * sequence (multiple of 64); position p lives in slot p % capacity, so a cache with capacity ==
  * window is the ring buffer the reference keeps for its sliding-window layers
- * (getp-csrc/src/alloc.cpp:245-250). */
-size_t gptoss_kv_cache_bytes(int B, int n_kv, int head_dim, int capacity); /* for K or V alone */
+ * (getp-csrc/src/alloc.cpp:245-250).  Sequences are the outermost dimension: the cache of the
+ * first n sequences is the first gptoss_kv_cache_bytes(n, ...) bytes. */
+size_t gptoss_kv_cache_bytes(int B, int n_kv, int head_dim, int capacity); /* K and V together */
 
 /* Store n_tok consecutive positions [pos0, pos0+n_tok) of every sequence.  k_rows/v_rows bf16
  * [B, n_tok, n_kv, head_dim] (K already rotated).  Bulk form of the cache write in
  * qkv_split_rope_store_kernel (layer_hip_batch.cpp:686-776). */
-int gptoss_kv_cache_write(void *k_cache, void *v_cache, const void *k_rows, const void *v_rows,
-                          int B, int n_kv, int head_dim, int capacity, int pos0, int n_tok,
-                          void *stream);
+int gptoss_kv_cache_write(void *kv_cache, const void *k_rows, const void *v_rows, int B, int n_kv,
+                          int head_dim, int capacity, int pos0, int n_tok, void *stream);
 
 size_t gptoss_attn_workspace_bytes(int B, int n_q, int n_kv, int head_dim, int max_len);
 
@@ -180,15 +183,15 @@ size_t gptoss_attn_workspace_bytes(int B, int n_q, int n_kv, int head_dim, int m
  *   positions; sinks fp32 [n_q] or NULL; out bf16 [B,n_q,D].
  *   max_len: upper bound of lens known to the host (sizes the split of long sequences).
  * Needs D in {32,64}, n_q % n_kv == 0, n_q/n_kv <= 16. */
-int gptoss_attn_decode(const float *q, const void *k_cache, const void *v_cache, const int *lens,
-                       const float *sinks, void *out, int B, int n_q, int n_kv, int head_dim,
-                       int capacity, int window, int max_len, void *workspace,
-                       size_t workspace_bytes, void *stream);
+int gptoss_attn_decode(const float *q, const void *kv_cache, const int *lens, const float *sinks,
+                       void *out, int B, int n_q, int n_kv, int head_dim, int capacity, int window,
+                       int max_len, void *workspace, size_t workspace_bytes, void *stream);
 
 /* gptoss_attn_decode for callers that cannot allocate or bring a workspace (code under HIP graph
  * capture, serving loops and harnesses that forbid hipMalloc).  No counterpart in the reference.
- * Same arguments, arithmetic and results as gptoss_attn_decode; the chunk partials of long
- * sequences go to a device array built into the library (64 MiB, held by every GPU the library
+ * Same arguments, arithmetic and results as gptoss_attn_decode; what that call keeps in its
+ * workspace (the chunk partials of long sequences when few sequences are served, the row order
+ * when many are) goes to a device array built into the library (64 MiB, held by every GPU the library
  * runs on until the process ends).  The call allocates nothing.  Refused with
  * GPTOSS_ERR_WORKSPACE when gptoss_attn_workspace_bytes(B, n_q, n_kv, head_dim, max_len) exceeds
  * gptoss_attn_decode_static_max_bytes() (e.g. 256 sequences x 64 heads x 64 up to 4096 positions
@@ -196,9 +199,9 @@ int gptoss_attn_decode(const float *q, const void *k_cache, const void *v_cache,
  * calls that overlap on one GPU (two streams, two threads) race; calls on one stream do not.  The
  * first call on a device looks the array's address up (make it outside a graph capture). */
 size_t gptoss_attn_decode_static_max_bytes(void);
-int gptoss_attn_decode_static(const float *q, const void *k_cache, const void *v_cache, const int *lens,
-                              const float *sinks, void *out, int B, int n_q, int n_kv, int head_dim,
-                              int capacity, int window, int max_len, void *stream);
+int gptoss_attn_decode_static(const float *q, const void *kv_cache, const int *lens, const float *sinks,
+                              void *out, int B, int n_q, int n_kv, int head_dim, int capacity, int window,
+                              int max_len, void *stream);
 
 /* The same attention for T consecutive positions of every sequence at once (prompt processing):
  * q fp32 [B, T, n_q, D] and out bf16 [B, T, n_q, D]; row (b, t) attends to the cached positions up
@@ -208,10 +211,9 @@ int gptoss_attn_decode_static(const float *q, const void *k_cache, const void *v
  * already hold positions [0, pos0 + T) of every sequence, all of them (a sliding-window ring
  * shorter than pos0 + T is refused: copy the prompt's K/V to a linear cache for this call). */
 size_t gptoss_attn_prefill_workspace_bytes(int B, int T, int n_q, int n_kv, int head_dim, int max_len);
-int gptoss_attn_prefill(const float *q, const void *k_cache, const void *v_cache, const float *sinks,
-                        void *out, int B, int T, int pos0, int n_q, int n_kv, int head_dim,
-                        int capacity, int window, void *workspace, size_t workspace_bytes,
-                        void *stream);
+int gptoss_attn_prefill(const float *q, const void *kv_cache, const float *sinks, void *out, int B,
+                        int T, int pos0, int n_q, int n_kv, int head_dim, int capacity, int window,
+                        void *workspace, size_t workspace_bytes, void *stream);
 
 /* ------------------------------------------------------------------ engine ------------------ */
 

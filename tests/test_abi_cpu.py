@@ -53,7 +53,7 @@ def test_no_oracle_or_cpu_fallback_in_product(lib):
 
 def test_argument_validation_without_gpu(lib):
     L = lib.load()
-    assert L.gptoss_abi_version() == 100
+    assert L.gptoss_abi_version() == 101
     # null pointers and bad dimensions are rejected before anything touches a device
     assert L.gptoss_router_gemm(None, None, None, None, 4, 256, 8, None) == 1
     assert "null" in lib.last_error()
@@ -65,8 +65,8 @@ def test_argument_validation_without_gpu(lib):
     assert L.gptoss_moe_route(p, 4, 32, 4, p, p, p, p, p, p, 100, None) == 2     # odd tile size
     assert L.gptoss_pack_weight(p, p, 1, 48, 64, 0, None) == 2                # n_out % 32
     assert L.gptoss_pack_weight(p, p, 1, 32, 100, lib.PACK_GLU, None) == 2    # n_in % 64
-    assert L.gptoss_kv_cache_write(p, p, p, p, 1, 2, 48, 64, 0, 1, None) == 2  # head_dim
-    assert L.gptoss_attn_decode(p, p, p, p, None, p, 1, 8, 3, 64, 64, 0, 10, p, 1 << 20, None) == 2
+    assert L.gptoss_kv_cache_write(p, p, p, 1, 2, 48, 64, 0, 1, None) == 2  # head_dim
+    assert L.gptoss_attn_decode(p, p, p, None, p, 1, 8, 3, 64, 64, 0, 10, p, 1 << 20, None) == 2
     w = lib.MoeWeights(32, 4, 2880, 2880, 7.0, p.value, p.value, p.value, p.value, p.value, p.value)
     assert L.gptoss_moe_forward(C.byref(w), p, 8, p, 0, None, 0, None) == 4   # no workspace
     assert "workspace" in lib.last_error()
@@ -74,7 +74,7 @@ def test_argument_validation_without_gpu(lib):
     assert L.gptoss_moe_forward(C.byref(w), p, 8, p, 0, p, 1 << 30, None) == 2
     # size queries are pure functions
     assert L.gptoss_packed_weight_bytes(32, 5760, 2880) == 32 * 5760 * 2880 * 2
-    assert L.gptoss_kv_cache_bytes(256, 8, 64, 4096) == 256 * 8 * 64 * 4096 * 2
+    assert L.gptoss_kv_cache_bytes(256, 8, 64, 4096) == 256 * 8 * 64 * 4096 * 2 * 2
     assert L.gptoss_moe_max_tiles(1024, 4, 32, 256) == 16 + 32
     assert L.gptoss_moe_workspace_bytes(1024, 32, 4, 2880, 2880) > 4096 * 2880 * 6
     assert L.gptoss_attn_workspace_bytes(256, 64, 8, 64, 4096) > 0
@@ -119,8 +119,8 @@ def test_engine_entry_points_validate_before_touching_a_device(lib):
     assert L.gptoss_engine_generate(None, p, p, 1, 1, 8, p, C.byref(n)) == 1
     assert L.gptoss_engine_generate_ragged(None, p, p, 1, 1, 8, None, p, C.byref(n)) == 1
     # prompt attention: shape checks come before any launch
-    assert L.gptoss_attn_prefill(p, p, p, None, p, 0, 4, 0, 8, 2, 32, 64, 0, p, 1 << 20, None) == 2      # B = 0
-    assert L.gptoss_attn_prefill(p, p, p, None, p, 1, 200, 0, 8, 2, 32, 128, 128, p, 1 << 20, None) == 2  # ring too short
+    assert L.gptoss_attn_prefill(p, p, None, p, 0, 4, 0, 8, 2, 32, 64, 0, p, 1 << 20, None) == 2      # B = 0
+    assert L.gptoss_attn_prefill(p, p, None, p, 1, 200, 0, 8, 2, 32, 128, 128, p, 1 << 20, None) == 2  # ring too short
     assert "windowed cache" in lib.last_error()
     assert L.gptoss_attn_prefill_workspace_bytes(0, 4, 8, 2, 32, 64) == 0
     assert L.gptoss_attn_prefill_workspace_bytes(2, 64, 8, 2, 32, 64) > 2 * 64 * 4

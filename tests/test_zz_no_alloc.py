@@ -15,8 +15,7 @@ def test_attn_decode_static_equals_attn_decode(ops):
     g = torch.Generator(device="cuda").manual_seed(41)
     B1, B2 = 200, 37
     cache = ops.KVCache(B1, n_kv, D, S)
-    cache.k.copy_(torch.randn(cache.k.numel(), device="cuda", generator=g).to(torch.bfloat16))
-    cache.v.copy_(torch.randn(cache.v.numel(), device="cuda", generator=g).to(torch.bfloat16))
+    cache.kv.copy_(torch.randn(cache.kv.numel(), device="cuda", generator=g).to(torch.bfloat16))
     sinks = torch.randn(n_q, device="cuda", generator=g)
     rng = np.random.default_rng(2)
     attn = ops.AttnDecode(B1, n_q, n_kv, D, S)
@@ -28,8 +27,7 @@ def test_attn_decode_static_equals_attn_decode(ops):
         lens_np[0] = hi
         lens = torch.from_numpy(lens_np).cuda()
         q = torch.randn(B, n_q, D, device="cuda", generator=g)
-        small = ops.KVCache(B, n_kv, D, S)
-        small.k, small.v = cache.k[: small.k.numel()], cache.v[: small.v.numel()]
+        small = cache.first(B)
         want = attn.forward(q, small, lens, sinks, window=window, max_len=hi)
         out = torch.full((B, n_q, D), float("nan"), dtype=torch.bfloat16, device="cuda")
         got = ops.attn_decode_static(q, small, lens, n_q, sinks, window=window, max_len=hi, out=out)
