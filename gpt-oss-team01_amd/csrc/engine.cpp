@@ -312,36 +312,6 @@ void rope_tables(const gptoss_config &c, int n_pos, std::vector<float> &cs, std:
     }
 }
 
-int dense_gemm(const bf16_t *A, const bf16_t *W, const float *bias, void *out, int epi, int B, int N,
-               int K, hipStream_t s, float *amax_val = nullptr, int *amax_idx = nullptr) {
-  GemmParams g{};
-  g.amax_val = amax_val;
-  g.amax_idx = amax_idx;
-  g.A = A;
-  g.W = W;
-  g.bias = bias;
-  g.out = out;
-  g.tiles = nullptr;
-  g.dense_rows = B;
-  g.N = N;
-  g.K = K;
-  g.n_col_tiles = gemm_col_tiles(N);
-  // Row tile: the smallest size that holds every row of a small batch; for larger batches 96 rows
-  // for the projections (few column tiles: more row tiles keep more CUs busy, fewer re-read the
-  // weights from L2 less often; 96 measured best for N = 2880..5120 at 1024 rows on MI355X) and
-  // 128 rows for the unembedding (hundreds of column tiles, MFMA-bound, 1024 = 8 full tiles).
-  static const int sizes[5] = {32, 64, 96, 128, 160};
-  int rpt = 160;
-  for (int i = 0; i < 5; i++)
-    if (B <= sizes[i]) {
-      rpt = sizes[i];
-      break;
-    }
-  if (B > 96) rpt = (g.n_col_tiles >= 64) ? 128 : 96;
-  if (B >= 2048) rpt = 160;  // a prompt pass: thousands of rows, every weight fragment feeds five MFMAs
-  return run_gemm(g, false, epi, rpt, cdiv(B, rpt), s);
-}
-
 // most rows (sequences x positions) one prompt-processing pass works on
 constexpr long long PREFILL_ROWS = 8192;
 
@@ -1107,6 +1077,17 @@ extern "C" int gptoss_engine_generate(gptoss_engine *e, const int *host_prompts,
                                       long long *n_generated) {
   return gptoss_engine_generate_ragged(e, host_prompts, host_n_prompt, prompt_stride, n_req, max_seq_len, nullptr,
                                        host_out, n_generated);
+}
+
+extern "C" int gptoss_rope_tables(const gptoss_config *cfg, int n_pos, float *host_cos, float *host_sin) {
+  GPTOSS_REQUIRE(cfg && host_cos && host_sin, GPTOSS_ERR_NULL, "rope_tables: null pointer");
+  GPTOSS_REQUIRE(n_pos > 0 && cfg->head_dim > 0 && cfg->head_dim % 2 == 0 && cfg->rope_theta > 0.f, GPTOSS_ERR_DIM,
+                 "rope_tables: bad dimensions (n_pos=%d head_dim=%d)", n_pos, cfg->head_dim);
+  std::vector<float> cs, sn;
+  rope_tables(*cfg, n_pos, cs, sn);
+  memcpy(host_cos, cs.data(), cs.size() * sizeof(float));
+  memcpy(host_sin, sn.data(), sn.size() * sizeof(float));
+  return GPTOSS_OK;
 }
 
 // Device view of one weight tensor in the layout the kernels read.

@@ -44,6 +44,9 @@ inline bool combine_norm_applies(int H, const float *norm_w, const bf16_t *norm_
 int moe_forward_norm(const gptoss_moe_weights *w, const void *t, int B, float *out, void *workspace,
                      size_t workspace_bytes, hipStream_t s, int mxfp4, const float *norm_w, bf16_t *norm_out);
 int moe_rows_per_tile(int B, int k, int E, bool mxfp4);
+// dense C = A . W^T (+ bias) with the epilogue `epi`; EPI_ARGMAX fills amax_val / amax_idx [B, gemm_col_tiles(N)]
+int dense_gemm(const bf16_t *A, const bf16_t *W, const float *bias, void *out, int epi, int B, int N, int K,
+               hipStream_t s, float *amax_val = nullptr, int *amax_idx = nullptr);
 int gemm_col_tiles(int N);  // column tiles of one workgroup's width
 // moe_route.hip
 int run_router(const void *t, const void *w_router, const float *b_router, float *logits, int B,

@@ -216,6 +216,7 @@ static int dispatch_rows(const GemmParams &p, int rows_per_tile, int max_tiles, 
 hipError_t gemm_set_attrs_bf16();   // gemm_bf16.hip
 hipError_t gemm_set_attrs_mxfp4();  // gemm_mxfp4.hip
 
+
 // Raises the dynamic-LDS limit of every GEMM kernel on the calling thread's current device, the
 // first time that device launches one.
 static int gemm_prepare_device() {
@@ -247,6 +248,37 @@ int run_gemm(const GemmParams &p, bool gather, int epi, int rows_per_tile, int m
   if (!gather && epi == EPI_ARGMAX && p.tiles == nullptr && p.amax_val && p.amax_idx)
     return dispatch_rows<false, EPI_ARGMAX>(p, rows_per_tile, max_tiles, s);
   return fail(GPTOSS_ERR_DIM, "run_gemm: unsupported combination (gather=%d epi=%d)", (int)gather, epi);
+}
+
+// C[B, N] = A[B, K] . W[N, K]^T (+ bias): the dense GEMMs of a step (QKV and output projections,
+// classifier), with the kernel and row tile chosen from the batch size.
+int dense_gemm(const bf16_t *A, const bf16_t *W, const float *bias, void *out, int epi, int B, int N,
+               int K, hipStream_t s, float *amax_val, int *amax_idx) {
+  GemmParams g{};
+  g.amax_val = amax_val;
+  g.amax_idx = amax_idx;
+  g.A = A;
+  g.W = W;
+  g.bias = bias;
+  g.out = out;
+  g.tiles = nullptr;
+  g.dense_rows = B;
+  g.N = N;
+  g.K = K;
+  g.n_col_tiles = gemm_col_tiles(N);
+  // Row tile: the smallest size that holds every row of a small batch; for larger batches 96 rows
+  // for the projections (few column tiles: more row tiles keep more CUs busy, fewer re-read the
+  // weights from L2 less often) and 128 rows for the unembedding (hundreds of column tiles).
+  static const int sizes[5] = {32, 64, 96, 128, 160};
+  int rpt = 160;
+  for (int i = 0; i < 5; i++)
+    if (B <= sizes[i]) {
+      rpt = sizes[i];
+      break;
+    }
+  if (B > 96) rpt = (g.n_col_tiles >= 64) ? 128 : 96;
+  if (B >= 2048) rpt = 160;  // a prompt pass: thousands of rows, every weight fragment feeds five MFMAs
+  return run_gemm(g, false, epi, rpt, cdiv(B, rpt), s);
 }
 
 int run_combine(const float *y2, const float *topk_w, const int *inv_perm, float *out, int B, int H,

@@ -82,6 +82,14 @@ SIGNATURES = {
     "gptoss_attn_decode": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _sz, _vp]),
     "gptoss_attn_decode_static_max_bytes": (_sz, []),
     "gptoss_attn_decode_static": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp]),
+    "gptoss_embedding": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
+    "gptoss_rmsnorm": (_i, [_vp, _vp, _vp, _vp, _i, _i, _vp]),
+    "gptoss_dense_gemm": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
+    "gptoss_classifier_argmax_workspace_bytes": (_sz, [_i, _i]),
+    "gptoss_classifier_argmax": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp, _sz, _vp]),
+    "gptoss_argmax": (_i, [_vp, _vp, _i, _i, _vp]),
+    "gptoss_rope_tables": (_i, [C.POINTER(Config), _i, _vp, _vp]),
+    "gptoss_rope_kv_store": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "gptoss_engine_create": (_i, [C.POINTER(Config), _vp, _i, _i, _i, C.c_uint64,
                                   C.POINTER(_vp)]),
     "gptoss_engine_step": (_i, [_vp, _vp, _i, _i, _vp]),

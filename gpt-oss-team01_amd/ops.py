@@ -220,6 +220,77 @@ class AttnPrefill:
         return out
 
 
+# ---- glue ops (names follow getp-csrc/include/layer_hip_batch.hpp) -------------------------------
+def embedding_lookup(table, tokens):
+    """table bf16 [V,H], tokens int32 [B] -> fp32 [B,H]."""
+    _need_gpu()
+    V, H = table.shape
+    x = torch.empty(tokens.numel(), H, dtype=torch.float32, device=table.device)
+    _l.check(_l.load().gptoss_embedding(_ptr(table), _ptr(tokens), _ptr(x), tokens.numel(), H, V, _stream()))
+    return x
+
+
+def rmsnorm(x, weight, residual=None):
+    """x fp32 [B,H] (updated in place by += residual when given) -> bf16 [B,H]."""
+    _need_gpu()
+    B, H = x.shape
+    t = torch.empty(B, H, dtype=torch.bfloat16, device=x.device)
+    _l.check(_l.load().gptoss_rmsnorm(_ptr(x), _ptr(residual), _ptr(weight), _ptr(t), B, H, _stream()))
+    return t
+
+
+def dense_gemm(a, w_packed, n_out, bias=None, out=None):
+    """a bf16 [B,K], w_packed = pack_weight(w [n_out,K]) -> fp32 [B,n_out]."""
+    _need_gpu()
+    B, K = a.shape
+    if out is None:
+        out = torch.empty(B, n_out, dtype=torch.float32, device=a.device)
+    _l.check(_l.load().gptoss_dense_gemm(_ptr(a), _ptr(w_packed), _ptr(bias), _ptr(out), B, n_out, K, _stream()))
+    return out
+
+
+def classifier_argmax(a, w_packed, vocab):
+    """arg max over the vocabulary of a . w^T without the logits: a bf16 [B,K] -> int32 [B]."""
+    _need_gpu()
+    L = _l.load()
+    B, K = a.shape
+    nb = L.gptoss_classifier_argmax_workspace_bytes(B, vocab)
+    ws = torch.empty(max(nb, 256), dtype=torch.uint8, device=a.device)
+    ids = torch.empty(B, dtype=torch.int32, device=a.device)
+    _l.check(L.gptoss_classifier_argmax(_ptr(a), _ptr(w_packed), _ptr(ids), B, vocab, K, _ptr(ws), nb, _stream()))
+    return ids
+
+
+def argmax(logits):
+    _need_gpu()
+    B, V = logits.shape
+    ids = torch.empty(B, dtype=torch.int32, device=logits.device)
+    _l.check(_l.load().gptoss_argmax(_ptr(logits), _ptr(ids), B, V, _stream()))
+    return ids
+
+
+def rope_tables(cfg, n_pos):
+    """-> (cos, sin) float32 numpy arrays [n_pos, head_dim/2] (host)."""
+    import numpy as np
+    cc = _l.Config.from_config(cfg)
+    cs = np.empty((n_pos, cfg.head_dim // 2), np.float32)
+    sn = np.empty_like(cs)
+    _l.check(_l.load().gptoss_rope_tables(C.byref(cc), n_pos, cs.ctypes.data_as(C.c_void_p),
+                                          sn.ctypes.data_as(C.c_void_p)))
+    return cs, sn
+
+
+def rope_kv_store(qkv, cache: KVCache, cos_t, sin_t, lens, n_q):
+    """qkv fp32 [B,(n_q+2n_kv)*D]; rotates q and k for position lens[b]-1, stores k, v into the cache;
+    -> q fp32 [B,n_q,D]."""
+    _need_gpu()
+    B = qkv.shape[0]
+    q = torch.empty(B, n_q, cache.D, dtype=torch.float32, device=qkv.device)
+    _l.check(_l.load().gptoss_rope_kv_store(_ptr(qkv), _ptr(q), _ptr(cache.kv), _ptr(cos_t), _ptr(sin_t),
+                                            _ptr(lens), B, n_q, cache.n_kv, cache.D, cache.cap, _stream()))
+    return q
+
+
 class KernelTrace:
     """Per-kernel HIP-event timing of the entry points called inside the ``with`` block
     (events are recorded on the stream each kernel is launched on)."""

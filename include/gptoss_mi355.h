@@ -215,8 +215,6 @@ int gptoss_attn_prefill(const float *q, const void *kv_cache, const float *sinks
                         int T, int pos0, int n_q, int n_kv, int head_dim, int capacity, int window,
                         void *workspace, size_t workspace_bytes, void *stream);
 
-/* ------------------------------------------------------------------ engine ------------------ */
-
 /* The 60-byte header of the flat .bin (reference run.cpp:25-45), same field order. */
 typedef struct {
   int vocab_size, hidden_dim, n_experts, experts_per_token, intermediate_dim, n_layers;
@@ -225,6 +223,56 @@ typedef struct {
   int sliding_window;
   float swiglu_limit;
 } gptoss_config;
+
+/* ------------------------------------------------------------------ glue ops ---------------- */
+/* The small ops between the two hot ones, for a host that keeps the reference's forward loop
+ * (getp-csrc/src/model.cpp:6-151) and binds it op by op; the engine below uses the same kernels. */
+
+/* x[b,:] = table[tokens[b],:]  (bf16 [V,H] row-major -> fp32 [B,H]; ids are clamped to 0..V-1).
+ * Replaces embedding_lookup_batched (getp-csrc/src/layer_hip_batch.cpp:199-242). */
+int gptoss_embedding(const void *table, const int *tokens, float *x, int B, int H, int V, void *stream);
+
+/* RMSNorm with the CPU model's arithmetic (run.cpp:304-317: double sum of squares, eps 1e-5 after
+ * the mean): t = weight * x / sqrt(mean(x^2) + eps) as bf16 [B,H].  With residual != NULL,
+ * x += residual first, in place.  Replaces rmsnorm_batched_quantize and
+ * residual_rmsnorm_batched_quantize (layer_hip_batch.cpp:339-438, 94-197). */
+int gptoss_rmsnorm(float *x, const float *residual, const float *weight, void *t_bf16, int B, int H,
+                   void *stream);
+
+/* out[B,N] = a[B,K] . w[N,K]^T + bias[N]   (bf16 x bf16 -> fp32; w in gptoss_pack_weight order; bias
+ * may be NULL).  Replaces qkv_gemm_batched_v2_quantize, attn_out_project_batched_v2_quantize and
+ * classifier_gemm_batched_v2_quantize (layer_hip_batch.cpp:644-683, 881-923, 1465-1501).
+ * Needs N % 32 == 0, K % 64 == 0, B*max(N,K) < 2^32. */
+int gptoss_dense_gemm(const void *a, const void *w_packed, const float *bias, float *out, int B, int N,
+                      int K, void *stream);
+
+/* next_ids[b] = arg max over v of a[b,:] . w[v,:]  (lowest v among equal maxima) without writing the
+ * [B,V] logits: the classifier GEMM keeps (max, column) per row and 256-column tile, a second small
+ * kernel picks the row's winner.  Replaces classifier_gemm_batched_v2_quantize + max_logits_batched
+ * (layer_hip_batch.cpp:1465-1501, 1542-1630; model.cpp:144-148). */
+size_t gptoss_classifier_argmax_workspace_bytes(int B, int V);
+int gptoss_classifier_argmax(const void *a, const void *w_packed, int *next_ids, int B, int V, int K,
+                             void *workspace, size_t workspace_bytes, void *stream);
+
+/* ids[b] = arg max of logits[b,:], lowest index among equal maxima (run.cpp:739-750).  Replaces
+ * max_logits_batched (layer_hip_batch.cpp:1542-1630).  Needs V % 4 == 0. */
+int gptoss_argmax(const float *logits, int *ids, int B, int V, void *stream);
+
+/* cos/sin tables [n_pos, head_dim/2] of the rotary embedding with YaRN scaling, the float arithmetic
+ * of run.cpp:404-478, written to HOST arrays.  Replaces rope_precompute_cs
+ * (getp-csrc/include/alloc.hpp:11-93). */
+int gptoss_rope_tables(const gptoss_config *cfg, int n_pos, float *host_cos, float *host_sin);
+
+/* Split the fused qkv rows [B,(n_q+2n_kv)*D] fp32, rotate q and k of sequence b for position
+ * lens[b]-1 (half-split pairs, run.cpp:480-499), write q fp32 [B,n_q,D] and store k, v as bf16 into
+ * slot (lens[b]-1) % capacity of the layer's cache.  cos_t / sin_t: DEVICE copies of the
+ * gptoss_rope_tables arrays covering every position used.  Replaces qkv_split_rope_fused
+ * (layer_hip_batch.cpp:686-816), with a position per sequence instead of one for the batch. */
+int gptoss_rope_kv_store(const float *qkv, float *q_out, void *kv_cache, const float *cos_t,
+                         const float *sin_t, const int *lens, int B, int n_q, int n_kv, int head_dim,
+                         int capacity, void *stream);
+
+/* ------------------------------------------------------------------ engine ------------------ */
 
 typedef struct gptoss_engine gptoss_engine;
 
