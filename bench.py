@@ -26,10 +26,32 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0         # MI355X HBM3E
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
-# HBM bytes of one GEMM1 launch at the default workload, from two rocprofv3 --pmc runs of this
-# command (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, the factors the 1 GiB copy below calibrates); the
-# summary is kept in profiles/moe_layer_20b_1024tok_and_decode_attention_kernel_stats_and_hbm_traffic.md
-GEMM1_HBM_TRAFFIC_BYTES = (1_101_846 + 23_041) * 1024
+GEMM1_KERNEL = "grouped_gemm_kernel<5, true, 1, false>"
+GEMM1_TRAFFIC_FILE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles",
+                                  "gemm1_bf16_20b_1024tok_hbm_traffic.txt")
+
+
+def measured_traffic(workload):
+    """HBM bytes of one launch of the roofline kernel, as two rocprofv3 --pmc runs of this command
+    counted them (FETCH_SIZE and WRITE_SIZE, each scaled by what it reads for the 1 GiB copy
+    below).  The figure is read from the committed counter summary and returned only if that
+    summary is for this kernel on this workload; otherwise None."""
+    try:
+        kv = {}
+        with open(GEMM1_TRAFFIC_FILE) as f:
+            for line in f:
+                if line.startswith("#") or ":" not in line:
+                    continue
+                k, v = line.split(":", 1)
+                kv[k.strip()] = v.strip()
+        if kv.get("kernel") != GEMM1_KERNEL:
+            return None
+        for k, v in workload.items():
+            if int(kv[k]) != int(v):
+                return None
+        return int(kv["traffic_bytes"])
+    except (OSError, KeyError, ValueError):
+        return None
 
 
 def parse():
@@ -492,10 +514,12 @@ def main():
                    "tokens": args.tokens, "hidden": 2880, "experts": 32, "top_k": 4,
                    "intermediate": 2880, "weights": "bf16 N(0,0.02), two sets alternated",
                    "activations": "bf16 N(0,1)"},
-        "roofline": {"kernel": "grouped_gemm_kernel<5,true,1,false> (gather + GEMM1 + SwiGLU)",
+        "roofline": {"kernel": GEMM1_KERNEL + " (gather + GEMM1 + SwiGLU)",
                      "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": GEMM1_HBM_TRAFFIC_BYTES if args.tokens == 1024 else None,
+                     "traffic": measured_traffic({"tokens": args.tokens, "hidden": 2880,
+                                                  "intermediate": 2880, "experts": 32,
+                                                  "top_k": 4}),
                      "bytes_per_launch": moe["gemm1_bytes"],
                      "avg_launch_us": round(moe["gemm1_ms"] * 1e3, 2)},
         "cpu_baseline": cpu,
