@@ -182,7 +182,12 @@ size_t gptoss_attn_workspace_bytes(int B, int n_q, int n_kv, int head_dim, int m
  *   reference has one scalar pos for the whole batch); window > 0 keeps the last `window`
  *   positions; sinks fp32 [n_q] or NULL; out bf16 [B,n_q,D].
  *   max_len: upper bound of lens known to the host (sizes the split of long sequences).
- * Needs D in {32,64}, n_q % n_kv == 0, n_q/n_kv <= 16. */
+ * Needs D in {32,64}, n_q % n_kv == 0, n_q/n_kv <= 16.
+ * A row's result does not depend on the other rows of the call, with one exception: a row that
+ * spans more than 512 slots is summed in one of two orders, chosen by the call's B * n_kv (below
+ * 512: chunks of 512 slots, merged by a second kernel; from 512 on: four interleaved streams merged
+ * inside one workgroup).  Calls with equal B, n_kv give bit-identical rows; across the two forms
+ * rows agree to fp32 rounding of the softmax sums. */
 int gptoss_attn_decode(const float *q, const void *kv_cache, const int *lens, const float *sinks,
                        void *out, int B, int n_q, int n_kv, int head_dim, int capacity, int window,
                        int max_len, void *workspace, size_t workspace_bytes, void *stream);
@@ -205,8 +210,8 @@ int gptoss_attn_decode_static(const float *q, const void *kv_cache, const int *l
 
 /* The same attention for T consecutive positions of every sequence at once (prompt processing):
  * q fp32 [B, T, n_q, D] and out bf16 [B, T, n_q, D]; row (b, t) attends to the cached positions up
- * to pos0 + t of sequence b, with the arithmetic gptoss_attn_decode uses for lens = pos0 + t + 1,
- * so its result is the one the T lock-step calls of the reference would give
+ * to pos0 + t of sequence b, with the arithmetic gptoss_attn_decode uses for lens = pos0 + t + 1
+ * and the same B, so its result is the one the T lock-step calls of the reference would give
  * (getp-csrc/submit/getp_run_submit.cpp:60-72 feeds prompts one position per step).  The cache must
  * already hold positions [0, pos0 + T) of every sequence, all of them (a sliding-window ring
  * shorter than pos0 + T is refused: copy the prompt's K/V to a linear cache for this call). */
