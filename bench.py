@@ -105,6 +105,27 @@ def bench_moe(ops, torch, args):
             layers[i % 2].forward(t, out)
     kern = trace.summary()
 
+    # the same layer under a skewed routing (what trained routers produce): a Zipf(1.1) bias over a
+    # fixed permutation of the experts replaces the router bias, then the original bias is restored
+    import numpy as np
+    ranks = np.random.default_rng(5).permutation(E) + 1
+    zipf = torch.from_numpy(np.log(1.0 / ranks ** 1.1).astype(np.float32)).to(dev)
+    saved = [l.b_router.clone() for l in layers]
+    for l in layers:
+        l.b_router.copy_(zipf)
+    for i in range(args.warmup):
+        layers[i % 2].forward(t, out)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        layers[i % 2].forward(t, out)
+    torch.cuda.synchronize()
+    ms_zipf = (time.perf_counter() - t0) * 1e3 / args.steps
+    counts = np.diff(layers[0].routing_views()[3].cpu().numpy())
+    for l, b in zip(layers, saved):
+        l.b_router.copy_(b)
+    torch.cuda.synchronize()
+
     flops = 2.0 * B * k * H * 3 * I + 2.0 * B * H * E
     w1_bytes = E * 2 * I * H * 2
     w2_bytes = E * H * I * 2
@@ -120,6 +141,10 @@ def bench_moe(ops, torch, args):
         "gemm1_ms": gemm1_ms,
         "gemm1_bytes": gemm1_bytes,
         "gemm1_flops": 2.0 * B * k * H * 2 * I,
+        "zipf": {"ms_per_step": round(ms_zipf, 5), "tokens_per_s": round(B / ms_zipf * 1e3, 1),
+                 "rows_per_expert": {"min": int(counts.min()), "max": int(counts.max()),
+                                     "above_160": int((counts > 160).sum())},
+                 "config": "same layer and tokens, router bias replaced by log(rank^-1.1)"},
     }
     return res, (raw[0], t, layers[0], out)
 
@@ -472,7 +497,8 @@ def main():
              "moe_weight_gbs": round(moe["weight_gbs"], 1),
              "moe_weight_hbm_frac": round(moe["weight_gbs"] / HBM_PEAK_GBS, 4),
              "moe_kernels_us": moe["kernels_us"],
-             "gemm1_tflops": round(moe["gemm1_flops"] / moe["gemm1_ms"] / 1e9, 1)}
+             "gemm1_tflops": round(moe["gemm1_flops"] / moe["gemm1_ms"] / 1e9, 1),
+             "moe_zipf_routing": moe["zipf"]}
     if attn is not None:
         extra["decode_attn"] = attn
         if args.cpu_tokens > 0:

@@ -6,6 +6,12 @@ namespace gptoss {
 
 enum { EPI_F32 = 0, EPI_SWIGLU = 1, EPI_BF16 = 2, EPI_ARGMAX = 3 };
 
+// Row tiles of ONE expert are grouped into blocks of up to MOE_TILE_BLOCK consecutive tiles by the
+// grouping kernel; a block never spans two experts, so every tile of a block multiplies the same
+// weights.
+constexpr int MOE_TILE_BLOCK = 8;
+constexpr int XCD_BOUNDS_INTS = 16;  // ints reserved for the cut positions in front of the block table
+
 struct GemmParams {
   const bf16_t *A;     // activations, row-major [*, K]
   const int *row_ids;  // gather: sorted pair ids (row of A = id / top_k); else unused
@@ -18,9 +24,11 @@ struct GemmParams {
   int *amax_idx;       // ... and the lowest column that holds it, [rows, n_col_tiles]
   const int *tiles;    // {n_tiles, (mat,row0,rows)*} or nullptr for a dense problem
   const int *xcd_bounds;  // 9 positions in the tile list (tile << 16 | 16-bit fraction) that cut the
-                          // work into 8 parts of equal estimated cost, or nullptr: equal item counts
-  int tile_block;      // grouped problems: row tiles that are walked together, column tile by column
-                       // tile (0 or 1 = every row tile on its own)
+                          // work into 8 parts of equal estimated cost, or nullptr: equal item counts.
+                          // From index XCD_BOUNDS_INTS on: one int per row tile, the block it belongs
+                          // to (first tile << 8 | tiles in the block; see MOE_TILE_BLOCK)
+  int tile_block;      // grouped problems, > 1: the row tiles of a block are walked together, column
+                       // tile by column tile (needs xcd_bounds); 0 or 1 = every row tile on its own
   int dense_rows;      // rows of the dense problem when tiles == nullptr
   int N, K;
   int n_col_tiles;     // gemm_col_tiles(N)
@@ -52,7 +60,7 @@ int gemm_col_tiles(int N);  // column tiles of one workgroup's width
 int run_router(const void *t, const void *w_router, const float *b_router, float *logits, int B,
                int H, int E, int k, float *topk_w, int *topk_i, hipStream_t s);
 int run_topk_softmax(const float *logits, int B, int E, int k, float *topk_w, int *topk_i, hipStream_t s);
-// xcd_bounds (optional, 9 ints): see GemmParams; tile_cost0_x2 = twice the fixed part of a tile's
+// xcd_bounds (optional, XCD_BOUNDS_INTS + max_tiles ints): see GemmParams; tile_cost0_x2 = twice the fixed part of a tile's
 // cost in units of one 32-row block of arithmetic (cost = fixed + number of 32-row blocks)
 int run_group(int B, int E, int k, float *topk_w, int *topk_i, int *expert_offsets,
               int *sorted_pair_ids, int *inv_perm, int *tiles, int rows_per_tile, int *xcd_bounds,

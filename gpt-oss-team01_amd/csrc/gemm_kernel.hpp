@@ -520,17 +520,17 @@ __global__ __launch_bounds__(GEMM_THREADS, (gemm_two_per_cu(MBMAX, FP4) ? 4 : 2)
     const int work = lo + jj;
     Item it;
     int tile;
-    if (p.tiles && p.tile_block > 1) {
-      // grouped, experts with several row tiles: blocks of tile_block consecutive row tiles (mostly
-      // one expert's) are walked column tile by column tile, so that the workgroups of an XCD
-      // share each W column tile among the block's row tiles as well as each row tile among a
-      // few column tiles
-      const int per_block = p.tile_block * p.n_col_tiles;
-      const int tb = work / per_block;
-      const int v = work - tb * per_block;
-      const int th = min(p.tile_block, n_tiles - tb * p.tile_block);
+    if (p.tiles && p.tile_block > 1 && p.xcd_bounds) {
+      // grouped, experts with several row tiles: the row tiles of one expert form blocks of up to
+      // MOE_TILE_BLOCK tiles (table behind the cut positions) that are walked column tile by
+      // column tile, so that the workgroups of an XCD share each column tile of the expert's
+      // weights among the block's row tiles as well as each row tile among a few column tiles.
+      // A block covers the work indices [first * n_col_tiles, (first + count) * n_col_tiles).
+      const int info = p.xcd_bounds[XCD_BOUNDS_INTS + work / p.n_col_tiles];
+      const int first = info >> 8, th = info & 255;
+      const int v = work - first * p.n_col_tiles;
       it.ct = v / th;
-      tile = tb * p.tile_block + (v - it.ct * th);
+      tile = first + (v - it.ct * th);
     } else if (p.tiles) {
       // grouped: column tiles of one row tile are neighbours (the tile's gathered rows stay in L2)
       tile = work / p.n_col_tiles;

@@ -290,6 +290,11 @@ __global__ __launch_bounds__(SORT_THREADS) void group_sort_kernel(
             tp[0] = e;
             tp[1] = off_ex[i] + t * rows_per_tile;
             tp[2] = min(rows_per_tile, cnt[i] - t * rows_per_tile);
+            // the block of up to MOE_TILE_BLOCK tiles of this expert that the tile belongs to
+            if (xcd_bounds != nullptr) {
+              const int b0 = t - t % MOE_TILE_BLOCK;
+              xcd_bounds[XCD_BOUNDS_INTS + tile_ex[i] + t] = ((tile_ex[i] + b0) << 8) | min(MOE_TILE_BLOCK, nt[i] - b0);
+            }
           }
         }
       }
