@@ -65,6 +65,9 @@ def parse():
     ap.add_argument("--no-attn", action="store_true", help="skip the decode-attention figures")
     ap.add_argument("--no-e2e", action="store_true", help="skip the end-to-end decode figure")
     ap.add_argument("--no-mxfp4", action="store_true", help="skip the 120B-shape MXFP4 MoE figure")
+    ap.add_argument("--no-zipf", action="store_true",
+                    help="skip the skewed-routing figure of the headline layer (profile runs: every "
+                         "launch of the roofline kernel is then the headline workload)")
     ap.add_argument("--no-sched", action="store_true", help="skip the scheduler leg of the end-to-end figure")
     return ap.parse_args()
 
@@ -105,26 +108,32 @@ def bench_moe(ops, torch, args):
             layers[i % 2].forward(t, out)
     kern = trace.summary()
 
-    # the same layer under a skewed routing (what trained routers produce): a Zipf(1.1) bias over a
-    # fixed permutation of the experts replaces the router bias, then the original bias is restored
-    import numpy as np
-    ranks = np.random.default_rng(5).permutation(E) + 1
-    zipf = torch.from_numpy(np.log(1.0 / ranks ** 1.1).astype(np.float32)).to(dev)
-    saved = [l.b_router.clone() for l in layers]
-    for l in layers:
-        l.b_router.copy_(zipf)
-    for i in range(args.warmup):
-        layers[i % 2].forward(t, out)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        layers[i % 2].forward(t, out)
-    torch.cuda.synchronize()
-    ms_zipf = (time.perf_counter() - t0) * 1e3 / args.steps
-    counts = np.diff(layers[0].routing_views()[3].cpu().numpy())
-    for l, b in zip(layers, saved):
-        l.b_router.copy_(b)
-    torch.cuda.synchronize()
+    zipf_res = None
+    if not args.no_zipf:
+        # the same layer under a skewed routing (what trained routers produce): a Zipf(1.1) bias over a
+        # fixed permutation of the experts replaces the router bias, then the original bias is restored
+        import numpy as np
+        ranks = np.random.default_rng(5).permutation(E) + 1
+        zipf = torch.from_numpy(np.log(1.0 / ranks ** 1.1).astype(np.float32)).to(dev)
+        saved = [l.b_router.clone() for l in layers]
+        for l in layers:
+            l.b_router.copy_(zipf)
+        for i in range(args.warmup):
+            layers[i % 2].forward(t, out)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(args.steps):
+            layers[i % 2].forward(t, out)
+        torch.cuda.synchronize()
+        ms_zipf = (time.perf_counter() - t0) * 1e3 / args.steps
+        counts = np.diff(layers[0].routing_views()[3].cpu().numpy())
+        for l, b in zip(layers, saved):
+            l.b_router.copy_(b)
+        torch.cuda.synchronize()
+        zipf_res = {"ms_per_step": round(ms_zipf, 5), "tokens_per_s": round(B / ms_zipf * 1e3, 1),
+                    "rows_per_expert": {"min": int(counts.min()), "max": int(counts.max()),
+                                        "above_160": int((counts > 160).sum())},
+                    "config": "same layer and tokens, router bias replaced by log(rank^-1.1)"}
 
     flops = 2.0 * B * k * H * 3 * I + 2.0 * B * H * E
     w1_bytes = E * 2 * I * H * 2
@@ -141,10 +150,7 @@ def bench_moe(ops, torch, args):
         "gemm1_ms": gemm1_ms,
         "gemm1_bytes": gemm1_bytes,
         "gemm1_flops": 2.0 * B * k * H * 2 * I,
-        "zipf": {"ms_per_step": round(ms_zipf, 5), "tokens_per_s": round(B / ms_zipf * 1e3, 1),
-                 "rows_per_expert": {"min": int(counts.min()), "max": int(counts.max()),
-                                     "above_160": int((counts > 160).sum())},
-                 "config": "same layer and tokens, router bias replaced by log(rank^-1.1)"},
+        "zipf": zipf_res,
     }
     return res, (raw[0], t, layers[0], out)
 
