@@ -266,18 +266,34 @@ int dense_gemm(const bf16_t *A, const bf16_t *W, const float *bias, void *out, i
   g.N = N;
   g.K = K;
   g.n_col_tiles = gemm_col_tiles(N);
-  // Row tile: the smallest size that holds every row of a small batch; for larger batches 96 rows
-  // for the projections (few column tiles: more row tiles keep more CUs busy, fewer re-read the
-  // weights from L2 less often) and 128 rows for the unembedding (hundreds of column tiles).
+  // Row tile.  Up to 96 rows: the smallest size that holds every row, so the weights are requested
+  // once.  A prompt pass (thousands of rows): 160 rows, every weight fragment feeds five MFMAs.  In
+  // between the launch is a handful of rounds of work items on 256 CUs, and an item of MB 32-row
+  // blocks takes (0.39 + 0.115 MB) us per 64-k slab (measured at 1024 rows: 0.50 / 0.64 / 0.76 /
+  // 0.85 us for 32 / 64 / 96 / 128 rows), so the tile that needs the least rounds x slab time wins:
+  // 96 rows for the QKV projection of 1024 rows (220 items, one round), 64 for the output
+  // projection (192 items instead of 132: 48 -> 41 us).
   static const int sizes[5] = {32, 64, 96, 128, 160};
   int rpt = 160;
-  for (int i = 0; i < 5; i++)
-    if (B <= sizes[i]) {
-      rpt = sizes[i];
-      break;
+  if (B <= 96) {
+    for (int i = 0; i < 5; i++)
+      if (B <= sizes[i]) {
+        rpt = sizes[i];
+        break;
+      }
+  } else if (B < 2048 && g.n_col_tiles >= 64) {
+    rpt = 128;  // the unembedding: hundreds of column tiles, measured best at 1024 rows
+  } else if (B < 2048) {
+    double best = 0.0;
+    for (int mb = 1; mb <= 5; mb++) {
+      const long long items = (long long)cdiv(B, 32 * mb) * g.n_col_tiles;
+      const double cost = (double)((items + 255) / 256) * (0.39 + 0.115 * mb);
+      if (mb == 1 || cost <= best) {  // ties go to the larger tile: fewer re-reads of the weights
+        best = cost;
+        rpt = 32 * mb;
+      }
     }
-  if (B > 96) rpt = (g.n_col_tiles >= 64) ? 128 : 96;
-  if (B >= 2048) rpt = 160;  // a prompt pass: thousands of rows, every weight fragment feeds five MFMAs
+  }
   return run_gemm(g, false, epi, rpt, cdiv(B, rpt), s);
 }
 
