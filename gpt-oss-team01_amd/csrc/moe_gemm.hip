@@ -10,6 +10,7 @@ namespace gptoss {
 // Weighted combine: out[b,:] (+)= sum over the token's k experts, in ascending expert order (the
 // order of the reference CPU loop, run.cpp:642-704), of w * y2[row of that pair].  Products and
 // sums are rounded separately, as that loop rounds them.
+template <int VPT>  // float4 chunks per thread: rows of at most 1024 * VPT floats (0: any length, a loop)
 __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ y2,
                                                       const float *__restrict__ topk_w,
                                                       const int *__restrict__ inv_perm,
@@ -32,7 +33,7 @@ __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ 
         int tr = rows[j]; rows[j] = rows[j + 1]; rows[j + 1] = tr;
         float tw = w[j]; w[j] = w[j + 1]; w[j + 1] = tw;
       }
-  for (int h = threadIdx.x * 4; h < H; h += 256 * 4) {
+  auto chunk = [&](int h) {
     f32x4 agg = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int s = 0; s < 8; s++) {
@@ -49,6 +50,16 @@ __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ 
       for (int q = 0; q < 4; q++) agg[q] = __fadd_rn(prev[q], agg[q]);
     }
     *op = agg;
+  };
+  if constexpr (VPT > 0) {
+    // unrolled: the loads of every chunk are in flight before the first sum needs one
+#pragma unroll
+    for (int i = 0; i < VPT; i++) {
+      const int h = (threadIdx.x + 256 * i) * 4;
+      if (h < H) chunk(h);
+    }
+  } else {
+    for (int h = threadIdx.x * 4; h < H; h += 256 * 4) chunk(h);
   }
 }
 
@@ -312,7 +323,9 @@ int run_combine(const float *y2, const float *topk_w, const int *inv_perm, float
   }
   {
     TraceScope ts("combine", s);
-    combine_kernel<<<B, 256, 0, s>>>(y2, topk_w, inv_perm, out, H, k, accumulate);
+    if (H <= 3072 && H > 2048) combine_kernel<3><<<B, 256, 0, s>>>(y2, topk_w, inv_perm, out, H, k, accumulate);
+    else if (H <= 1024) combine_kernel<1><<<B, 256, 0, s>>>(y2, topk_w, inv_perm, out, H, k, accumulate);
+    else combine_kernel<0><<<B, 256, 0, s>>>(y2, topk_w, inv_perm, out, H, k, accumulate);
   }
   GPTOSS_LAUNCH_CHECK("combine_kernel");
   return GPTOSS_OK;
