@@ -41,7 +41,8 @@ constexpr float NEG_BIG = -1.0e30f;
 struct AttnParams {
   const float *q;      // [B, n_q, D]
   const bf16_t *kv;    // [B, n_kv, cap/64] blocks of K [64, D] + V [2, D/16, 64, 8]
-  const int *lens;     // [B]
+  const int *lens;     // [B], or nullptr: row b has len_base + b % len_period positions (len_period 0: len_base)
+  int len_base, len_period;
   const float *sinks;  // [n_q] or nullptr
   bf16_t *out;         // [B, n_q, D]
   float *part_o;       // [B, max_chunks, n_q, D]
@@ -54,6 +55,13 @@ struct AttnParams {
   int2 *order_out;     // chunked kernels: when set, one extra workgroup (the last) writes that order
   int order_buckets;   // slot-span buckets (of 64 slots) the order distinguishes
 };
+
+// Cached positions of query row b: the caller's array, or the rule a host that knows every length
+// passes instead (lock-step decoding: one length; a prompt pass: position within the sequence), which
+// saves the kernels a dependent load.
+__device__ __forceinline__ int row_len(const AttnParams &p, int b) {
+  return p.lens ? p.lens[b] : p.len_base + (p.len_period > 0 ? b % p.len_period : 0);
+}
 
 struct SeqRange {
   int s_begin, s_end;  // slot range to visit (s_begin is a multiple of 64)
@@ -103,7 +111,7 @@ __device__ __forceinline__ void attn_write_order(const AttnParams &p, int *hist 
     const SeqRange r = seq_range(len, p.cap, p.window, p.max_len);
     return r.nchunks > 1 ? min(nbk - 1, (r.s_end - r.s_begin + ATT_BLOCK - 1) / ATT_BLOCK) : 0;
   };
-  for (int b = tid; b < p.B; b += 256) atomicAdd(&hist[key_of(p.lens[b])], 1);
+  for (int b = tid; b < p.B; b += 256) atomicAdd(&hist[key_of(row_len(p, b))], 1);
   __syncthreads();
   // start[k] = number of rows with a larger key; thread t owns `per` consecutive buckets from the top
   const int per = (nbk + 255) / 256;
@@ -131,7 +139,7 @@ __device__ __forceinline__ void attn_write_order(const AttnParams &p, int *hist 
   }
   __syncthreads();
   for (int b = tid; b < p.B; b += 256) {
-    const int len = p.lens[b];
+    const int len = row_len(p, b);
     const int pos = atomicAdd(&start[key_of(len)], 1);
     p.order_out[pos] = make_int2(b, len);
   }
@@ -182,7 +190,7 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
   // the chip is still filling and the grid ends on chunk 0, which every sequence has
   const int chunk_id = WG ? 0 : p.max_chunks - 1 - rest / units;
   if (chunk_id < 0) return;
-  SeqRange r = seq_range((WG && p.order) ? ordered.y : __builtin_amdgcn_readfirstlane(p.lens[b]), p.cap, p.window,
+  SeqRange r = seq_range((WG && p.order) ? ordered.y : __builtin_amdgcn_readfirstlane(row_len(p, b)), p.cap, p.window,
                          p.max_len);
   if (WG) {
     if (r.nchunks <= 1) return;   // the whole workgroup: such rows belong to the one-wave kernel
@@ -190,7 +198,7 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
   }
   // the second row of a pair: the next row of the same sequence, when there is one
   const bool two = PAIR && 2 * pair_idx + 1 < p.rows_per_seq;
-  const SeqRange r1 = two ? seq_range(__builtin_amdgcn_readfirstlane(p.lens[b + 1]), p.cap, p.window, p.max_len) : r;
+  const SeqRange r1 = two ? seq_range(__builtin_amdgcn_readfirstlane(row_len(p, b + 1)), p.cap, p.window, p.max_len) : r;
   const bool act0 = WG || (chunk_id < r.nchunks && !(p.only_single && r.nchunks > 1));
   const bool act1 = two && chunk_id < r1.nchunks && !(p.only_single && r1.nchunks > 1);
   if (!act0 && !act1) return;
@@ -475,7 +483,7 @@ __global__ __launch_bounds__(256) void attn_reduce_kernel(AttnParams p) {
   const int d4 = (threadIdx.x % TPP) * 4;
   if (pair >= p.B * p.n_q) return;
   const int b = pair / p.n_q, hq = pair - b * p.n_q;
-  const SeqRange r = seq_range(p.lens[b], p.cap, p.window, p.max_len);
+  const SeqRange r = seq_range(row_len(p, b), p.cap, p.window, p.max_len);
   if (r.nchunks <= 1) return;  // already finished by the first kernel
   const float sink2 = p.sinks ? p.sinks[hq] * 1.4426950408889634f : -INFINITY;
   const size_t slot0 = (size_t)b * p.max_chunks * p.n_q + hq;
@@ -603,11 +611,13 @@ extern "C" size_t gptoss_attn_workspace_bytes(int B, int n_q, int n_kv, int head
 }
 
 // B query rows; row b reads the cache of sequence b / rows_per_seq up to its own lens[b]
+// (lens == nullptr: row b has len_base + b % len_period positions)
 static int attn_launch(const float *q, const void *kv_cache, const int *lens,
                        const float *sinks, void *out, int B, int rows_per_seq, int n_q, int n_kv,
                        int head_dim, int capacity, int window, int max_len, void *workspace,
-                       size_t workspace_bytes, void *stream) {
-  GPTOSS_REQUIRE(q && kv_cache && lens && out, GPTOSS_ERR_NULL, "attn_decode: null pointer");
+                       size_t workspace_bytes, void *stream, int len_base = 0, int len_period = 0) {
+  GPTOSS_REQUIRE(q && kv_cache && out, GPTOSS_ERR_NULL, "attn_decode: null pointer");
+  if (!lens && len_base == 0) len_base = max_len;  // no lengths given: every row has max_len positions
   GPTOSS_REQUIRE(B > 0 && n_q > 0 && n_kv > 0 && n_q % n_kv == 0 && n_q / n_kv <= 16, GPTOSS_ERR_DIM,
                  "attn_decode: need n_q %% n_kv == 0 and n_q/n_kv <= 16 (n_q=%d n_kv=%d)", n_q, n_kv);
   GPTOSS_REQUIRE(head_dim == 32 || head_dim == 64, GPTOSS_ERR_DIM,
@@ -630,6 +640,8 @@ static int attn_launch(const float *q, const void *kv_cache, const int *lens,
   p.q = q;
   p.kv = (const bf16_t *)kv_cache;
   p.lens = lens;
+  p.len_base = len_base;
+  p.len_period = len_period;
   p.sinks = sinks;
   p.out = (bf16_t *)out;
   int2 *order = (int2 *)workspace;
@@ -741,11 +753,6 @@ extern "C" int gptoss_attn_decode_static(const float *q, const void *kv_cache, c
                      ATTN_STATIC_SCRATCH_BYTES, stream);
 }
 
-__global__ __launch_bounds__(256) void prefill_lens_kernel(int *lens, int rows, int T, int pos0) {
-  const int r = blockIdx.x * 256 + threadIdx.x;
-  if (r < rows) lens[r] = pos0 + r % T + 1;
-}
-
 extern "C" size_t gptoss_attn_prefill_workspace_bytes(int B, int T, int n_q, int n_kv, int head_dim,
                                                       int max_len) {
   if (B <= 0 || T <= 0) return 0;
@@ -766,9 +773,8 @@ extern "C" int gptoss_attn_prefill(const float *q, const void *kv_cache, const f
   const size_t lens_bytes = align_up((size_t)rows * sizeof(int), 256);
   GPTOSS_REQUIRE(workspace && aligned(workspace, 256) && workspace_bytes > lens_bytes, GPTOSS_ERR_WORKSPACE,
                  "attn_prefill: workspace missing, misaligned or too small");
-  int *lens = (int *)workspace;
-  prefill_lens_kernel<<<(rows + 255) / 256, 256, 0, (hipStream_t)stream>>>(lens, rows, T, pos0);
-  GPTOSS_LAUNCH_CHECK("prefill_lens_kernel");
-  return attn_launch(q, kv_cache, lens, sinks, out, rows, T, n_q, n_kv, head_dim, capacity, window,
-                     pos0 + T, (unsigned char *)workspace + lens_bytes, workspace_bytes - lens_bytes, stream);
+  // row (b, t) has pos0 + t + 1 positions: a rule the kernels evaluate, no array of lengths
+  return attn_launch(q, kv_cache, nullptr, sinks, out, rows, T, n_q, n_kv, head_dim, capacity, window,
+                     pos0 + T, (unsigned char *)workspace + lens_bytes, workspace_bytes - lens_bytes, stream,
+                     pos0 + 1, T);
 }

@@ -711,8 +711,6 @@ static int step_impl(gptoss_engine *e, const int *host_tokens, int pos, const in
   if (host_pos) {
     for (int i = 0; i < B; i++) e->h_lens[i] = host_pos[i] + 1;
     GPTOSS_HIP(hipMemcpyAsync(e->d_lens, e->h_lens, sizeof(int) * B, hipMemcpyHostToDevice, s));
-  } else {
-    STEP(run_fill_int(e->d_lens, B, pos + 1, s));
   }
   STEP(run_embedding(e->embedding, e->d_tokens, e->x, B, H, V, s));
   for (int l = 0; l < L; l++) {
@@ -725,7 +723,8 @@ static int step_impl(gptoss_engine *e, const int *host_tokens, int pos, const in
     else
       STEP(run_rope_store(e->qkv, e->q, w.kv_cache, e->cos_t, e->sin_t, B, nq, nkv, D,
                           w.cache_cap, pos, s));
-    STEP(gptoss_attn_decode(e->q, w.kv_cache, e->d_lens, w.sinks, e->attn_out, B, nq, nkv, D,
+    // lock step: every sequence has pos + 1 positions, which the call takes from max_len
+    STEP(gptoss_attn_decode(e->q, w.kv_cache, host_pos ? e->d_lens : nullptr, w.sinks, e->attn_out, B, nq, nkv, D,
                             w.cache_cap, w.window, pos + 1, e->attn_ws, e->attn_ws_bytes, s));
     STEP(dense_gemm(e->attn_out, w.w_o, w.b_o, e->tb2, EPI_F32, B, H, nq * D, s));
     // x += attention branch, then the ffn norm (model.cpp:66)

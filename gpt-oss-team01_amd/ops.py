@@ -174,7 +174,7 @@ class AttnDecode:
 
     def forward(self, q, cache: KVCache, lens, sinks=None, window=0, out=None, max_len=None):
         B = q.shape[0]
-        assert q.dtype == torch.float32 and q.is_contiguous() and lens.dtype == torch.int32
+        assert q.dtype == torch.float32 and q.is_contiguous() and (lens is None or lens.dtype == torch.int32)
         if out is None:
             out = torch.empty(B, self.n_q, self.D, dtype=torch.bfloat16, device=q.device)
         _l.check(self.L.gptoss_attn_decode(_ptr(q), _ptr(cache.kv), _ptr(lens),

@@ -179,7 +179,8 @@ size_t gptoss_attn_workspace_bytes(int B, int n_q, int n_kv, int head_dim, int m
 /* Single-query attention with sinks and optional sliding window over the bf16 KV cache.
  * Replaces single_query_attn_flash_batched_quantize (getp-csrc/src/flash_attn_hip.cpp:847-923).
  *   q fp32 [B,n_q,D] (rotated); lens int32 [B] = cached positions per sequence (pos+1; the
- *   reference has one scalar pos for the whole batch); window > 0 keeps the last `window`
+ *   reference has one scalar pos for the whole batch), or NULL when every sequence has max_len
+ *   positions (lock-step decoding: the kernels then need no load to learn a row's length); window > 0 keeps the last `window`
  *   positions; sinks fp32 [n_q] or NULL; out bf16 [B,n_q,D].
  *   max_len: upper bound of lens known to the host (sizes the split of long sequences).
  * Needs D in {32,64}, n_q % n_kv == 0, n_q/n_kv <= 16.

@@ -112,6 +112,21 @@ def test_attn_len1_closed_form(ops):
             np.testing.assert_allclose(got[b, h], w * Vf[b, 0, g], rtol=1e-2, atol=1e-2)
 
 
+def test_attn_without_lengths_means_every_row_has_max_len(ops):
+    """lens = NULL (lock-step decoding: the host knows the one length) gives the bits of an array filled
+    with max_len, in both launch forms."""
+    for B, n_q, n_kv, D, S, L in ((5, 8, 2, 32, 256, 200), (70, 64, 8, 64, 640, 601)):
+        q, K, V, sinks = _mk(B, S, n_q, n_kv, D, seed=21)
+        cache = ops.KVCache(B, n_kv, D, S)
+        cache.write(K.cuda(), V.cuda(), 0)
+        attn = ops.AttnDecode(B, n_q, n_kv, D, S)
+        lens = torch.full((B,), L, dtype=torch.int32, device="cuda")
+        for window in (0, 128):
+            a = attn.forward(q.cuda(), cache, lens, sinks.cuda(), window=window, max_len=L).clone()
+            b = attn.forward(q.cuda(), cache, None, sinks.cuda(), window=window, max_len=L)
+            assert torch.equal(a, b), (B, window)
+
+
 def test_attn_bad_arguments(ops):
     import ctypes as C
     from conftest import load_pkg
