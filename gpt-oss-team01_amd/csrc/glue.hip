@@ -202,11 +202,6 @@ __global__ __launch_bounds__(256) void f32_to_bf16_kernel(const float *__restric
     dst[i] = f32_to_bf16(src[i]);
 }
 
-__global__ __launch_bounds__(256) void fill_int_kernel(int *__restrict__ dst, int n, int value) {
-  int i = blockIdx.x * 256 + threadIdx.x;
-  if (i < n) dst[i] = value;
-}
-
 // N(mean, std) from a counter-based generator (splitmix64 of seed+index, Box-Muller), rounded to
 // bf16 or kept fp32.  Used to build random-init models of sizes whose fp32 file would not fit.
 __device__ __forceinline__ uint64_t splitmix64(uint64_t z) {
@@ -421,12 +416,6 @@ int run_argmax(const float *logits, int *ids, int B, int V, hipStream_t s) {
 int run_f32_to_bf16(const float *src, bf16_t *dst, size_t n, hipStream_t s) {
   f32_to_bf16_kernel<<<grid_for(n), 256, 0, s>>>(src, dst, n);
   GPTOSS_LAUNCH_CHECK("f32_to_bf16_kernel");
-  return GPTOSS_OK;
-}
-
-int run_fill_int(int *dst, int n, int value, hipStream_t s) {
-  fill_int_kernel<<<cdiv(n, 256), 256, 0, s>>>(dst, n, value);
-  GPTOSS_LAUNCH_CHECK("fill_int_kernel");
   return GPTOSS_OK;
 }
 

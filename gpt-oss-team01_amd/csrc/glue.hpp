@@ -25,7 +25,6 @@ int run_gather_rows(const float *src, float *dst, int rows, int n, int stride, i
 int run_argmax(const float *logits, int *ids, int B, int V, hipStream_t s);
 int run_argmax_tiles(const float *val, const int *idx, int *ids, int B, int n_tiles, hipStream_t s);
 int run_f32_to_bf16(const float *src, bf16_t *dst, size_t n, hipStream_t s);
-int run_fill_int(int *dst, int n, int value, hipStream_t s);
 // fp32 [n_blocks * 32] -> e2m1 codes [n_blocks, 16] + e8m0 scales [n_blocks]; *not_exact is set when a
 // value has no exact MXFP4 representation
 int run_requant_mxfp4(const float *src, size_t n_blocks, unsigned char *blocks, unsigned char *scales,
