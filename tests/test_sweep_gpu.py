@@ -1,0 +1,164 @@
+"""Randomised shapes and model configurations (fixed seeds): the MoE layer, decode attention and the
+engine against the CPU oracle on dimensions no hand-picked case covers - odd token counts, one to 64
+experts, top-1 to top-8, skewed routing, every supported head grouping, ring caches that have
+wrapped, ragged lengths with empty rows."""
+import numpy as np
+import pytest
+import torch
+
+from conftest import TOL_MAX, TOL_MEAN, rel_errors
+
+pytestmark = pytest.mark.gpu
+
+
+def test_moe_random_shapes(ops, orc):
+    rng = np.random.default_rng(20240)
+    worst = [0.0, 0.0]
+    for case in range(48):
+        E = int(rng.choice([1, 2, 4, 8, 16, 32, 40, 64]))
+        k = int(min(E, rng.choice([1, 2, 4, 4, 4, 8])))
+        H = int(rng.choice([64, 128, 192, 256, 320, 512]))
+        I = int(rng.choice([64, 128, 192, 256, 384]))
+        B = int(rng.choice([1, 2, 3, 17, 31, 33, 64, 100, 129, 257, 500, 1000, 1500]))
+        skew = float(rng.choice([0.0, 0.0, 1.0, 3.0]))
+        g = torch.Generator().manual_seed(int(rng.integers(1 << 30)))
+        n = lambda *s: (torch.randn(*s, generator=g) * 0.05).to(torch.bfloat16)
+        br = (n(E).float() - skew * torch.arange(E) / max(E, 1)).to(torch.bfloat16)   # skew: a few hot experts
+        L = dict(w_router=n(E, H), b_router=br, w1=n(E, 2 * I, H), b1=n(E, 2 * I), w2=n(E, H, I), b2=n(E, H))
+        names = ("w_router", "b_router", "w1", "b1", "w2", "b2")
+        t = torch.randn(B, H, generator=g).to(torch.bfloat16)
+        layer = ops.MoeLayer(*[L[x].cuda() for x in names], top_k=k, max_tokens=B)
+        out = layer.forward(t.cuda()).clone()
+        assert torch.equal(out, layer.forward(t.cuda())), (case, "not reproducible")
+        logits, tw, ti, off, srt, inv = [x.cpu().numpy() for x in layer.routing_views()]
+        f = lambda x: x.float().cpu().numpy()
+        want, _, _, oti = orc.moe_layer(f(t), *[f(L[x]) for x in names], k=k, limit=7.0,
+                                        stage=orc.STAGE_SWIGLU, want_routing=True)
+        _, oi = orc.topk_softmax(logits, k)
+        ooff, osrt, oinv = orc.group(oi, E)
+        assert np.array_equal(ti, oi) and np.array_equal(off, ooff), case
+        assert np.array_equal(srt, osrt) and np.array_equal(inv, oinv), case
+        same = (oti == ti).all(axis=1)           # near-ties of the router may go the other way
+        assert same.mean() > 0.9, (case, same.mean())
+        if same.any():
+            mx, mean = rel_errors(out.cpu().numpy()[same], want[same])
+            worst = [max(worst[0], mx), max(worst[1], mean)]
+            assert mx <= TOL_MAX and mean <= TOL_MEAN, (case, E, k, H, I, B, mx, mean)
+    print("random MoE shapes: worst max-rel / mean-rel", worst)
+
+
+def test_attn_random_shapes(ops, orc):
+    rng = np.random.default_rng(20241)
+    worst = [0.0, 0.0]
+    for case in range(64):
+        D = int(rng.choice([32, 64]))
+        n_kv = int(rng.choice([1, 2, 4, 8]))
+        n_q = n_kv * int(rng.choice([1, 2, 4, 8, 16]))
+        B = int(rng.choice([1, 2, 5, 16, 63, 64, 65, 130]))
+        cap = int(rng.choice([64, 128, 192, 512, 1024, 2048]))
+        window = int(rng.choice([0, 0, 16, 64, 128, 200]))
+        wrapped = 0 < window <= cap and rng.random() < 0.4
+        max_len = int(rng.integers(cap + 1, 3 * cap)) if wrapped else int(rng.integers(1, cap + 1))
+        # a ring holds the last positions written, so every row of a wrapped cache is at the end
+        lens = np.full(B, max_len, np.int32) if wrapped else rng.integers(0, max_len + 1, size=B).astype(np.int32)
+        g = torch.Generator().manual_seed(int(rng.integers(1 << 30)))
+        q = torch.randn(B, n_q, D, generator=g)
+        K = torch.randn(B, max_len, n_kv, D, generator=g).to(torch.bfloat16)
+        V = torch.randn(B, max_len, n_kv, D, generator=g).to(torch.bfloat16)
+        sinks = torch.randn(n_q, generator=g)
+        cache = ops.KVCache(B, n_kv, D, cap)
+        cache.kv.view(torch.int16).fill_(0x7FC1)
+        for p0 in range(0, max_len, cap):
+            m = min(cap, max_len - p0)
+            cache.write(K[:, p0:p0 + m].contiguous().cuda(), V[:, p0:p0 + m].contiguous().cuda(), p0)
+        attn = ops.AttnDecode(B, n_q, n_kv, D, max_len)
+        got = attn.forward(q.cuda(), cache, torch.as_tensor(lens).cuda(), sinks.cuda(),
+                           window=window).float().cpu().numpy()
+        want = orc.attn_decode(q.numpy(), K.float().numpy(), V.float().numpy(), lens, sinks.numpy(), window)
+        live = lens > 0
+        if live.any():
+            assert np.isfinite(got[live]).all(), case
+            mx, mean = rel_errors(got[live], want[live])
+            worst = [max(worst[0], mx), max(worst[1], mean)]
+            assert mx <= TOL_MAX and mean <= TOL_MEAN, (case, B, n_q, n_kv, D, cap, window, max_len, mx, mean)
+    print("random attention shapes: worst max-rel / mean-rel", worst)
+
+
+def test_engine_random_configs(ops, orc, binfmt):
+    """Lock-step steps against the CPU model that rounds where the GPU dataflow rounds (rows are
+    dropped once a router decision comes closer than 1.5e-2: the two may then pick different
+    experts), the prompt pass against the lock-step steps (bit for bit while no sliding-window ring
+    has wrapped), and one step with per-sequence positions."""
+    rng = np.random.default_rng(20242)
+    done = 0
+    worst = 0.0
+    while done < 10:
+        D = int(rng.choice([32, 64]))
+        nkv = int(rng.choice([1, 2, 4]))
+        nq = nkv * int(rng.choice([1, 2, 4, 8]))
+        H = int(rng.choice([128, 192, 256, 320]))
+        E = int(rng.choice([4, 8, 16, 32]))
+        k = int(min(E, rng.choice([1, 2, 4])))
+        I = int(rng.choice([64, 128, 192, 256]))
+        L = int(rng.choice([1, 2, 3]))
+        V = int(rng.choice([256, 512, 1088, 1024, 4096]))
+        win = int(rng.choice([64, 128]))
+        seed = int(rng.integers(1 << 30))
+        B = int(rng.choice([1, 3, 8, 33]))
+        T = int(rng.choice([3, 9, 70 if win == 64 else 20]))
+        if ((nq + 2 * nkv) * D) % 64 or (nq * D) % 64:
+            continue                                         # the engine wants these multiples of 64
+        cfg = binfmt.Config(vocab_size=V, hidden_dim=H, n_experts=E, experts_per_token=k, intermediate_dim=I,
+                            n_layers=L, head_dim=D, n_attn_heads=nq, n_kv_heads=nkv, seq_len=2048,
+                            initial_context_length=4096, rope_theta=150000.0, rope_scaling_factor=32.0,
+                            sliding_window=win, swiglu_limit=7.0)
+        g = np.random.default_rng(seed)
+        flat = np.empty(binfmt.n_weight_floats(cfg), np.float32)
+        off = 0
+        for name, shape in binfmt.tensor_shapes(cfg).items():
+            m = int(np.prod(shape))
+            x = g.standard_normal(m).astype(np.float32) * 0.05
+            if name in ("attn_norm", "mlp_norm", "final_norm"):
+                x = x * 0.4 + 1.0
+            flat[off:off + m] = torch.from_numpy(x).to(torch.bfloat16).float().numpy()
+            off += m
+        toks = g.integers(0, V, size=(B, T + 1)).astype(np.int32)
+        a = ops.Engine(cfg, flat, max_batch=B, max_seq=128, keep_logits=True)
+        b = ops.Engine(cfg, flat, max_batch=B, max_seq=128, keep_logits=True)
+        rows = sorted({0, B // 2, B - 1})
+        cpu = {r: orc.Model(cfg, flat, stage=orc.STAGE_GPU) for r in rows}
+        live = set(rows)
+        for pos in range(T):
+            ids = a.step(toks[:, pos], pos)
+            got = a.last_logits(B)
+            assert np.array_equal(ids, got.argmax(axis=1)), (done, pos)
+            for r in rows:
+                want = cpu[r].forward(int(toks[r, pos]), pos)
+                if cpu[r].last_router_gap() < 1.5e-2:
+                    live.discard(r)
+                if r in live:
+                    mx, _ = rel_errors(got[r], want)
+                    worst = max(worst, mx)
+                    assert mx <= 2e-2, (done, pos, r, mx, cfg)
+        b.prefill(toks[:, :T])
+        lb = b.last_logits(B)
+        if T <= win:
+            assert np.array_equal(lb, got), (done, "prompt pass differs from lock step", cfg)
+        else:
+            per = np.abs(lb - got).max(axis=1) / np.abs(got).max(axis=1)
+            assert np.median(per) <= 5e-3, (done, per, cfg)
+        posv = np.array([T - (i % 2) for i in range(B)], np.int32)   # every other row repeats its last position
+        a.step_ragged(np.array([toks[i, posv[i]] for i in range(B)], np.int32), posv)
+        lr = a.last_logits(B)
+        for r in rows:
+            if r in live and posv[r] == T:
+                want = cpu[r].forward(int(toks[r, T]), T)
+                if cpu[r].last_router_gap() >= 1.5e-2:
+                    mx, _ = rel_errors(lr[r], want)
+                    assert mx <= 2e-2, (done, "ragged", r, mx, cfg)
+        a.close()
+        b.close()
+        for m in cpu.values():
+            m.close()
+        done += 1
+    print("random engine configurations: worst max-rel against the staged CPU model", worst)
