@@ -8,6 +8,7 @@
 #include <string.h>
 
 #include <algorithm>
+#include <system_error>
 #include <thread>
 #include <vector>
 
@@ -112,12 +113,20 @@ static void host_copy(float *dst, const float *src, size_t n) {
   }
   std::thread th[T - 1];
   const size_t per = (n + T - 1) / T;
+  int started = 0;
   for (int i = 1; i < T; i++) {
     const size_t lo = std::min(n, per * i), hi = std::min(n, per * (i + 1));
-    th[i - 1] = std::thread([=] { memcpy(dst + lo, src + lo, (hi - lo) * sizeof(float)); });
+    try {
+      th[i - 1] = std::thread([=] { memcpy(dst + lo, src + lo, (hi - lo) * sizeof(float)); });
+      started = i;
+    } catch (const std::system_error &) {
+      break;  // no more threads to be had (a thread or pid limit): this thread copies the rest
+    }
   }
   memcpy(dst, src, std::min(n, per) * sizeof(float));
-  for (int i = 1; i < T; i++) th[i - 1].join();
+  const size_t rest = std::min(n, per * (size_t)(started + 1));
+  if (rest < n) memcpy(dst + rest, src + rest, (n - rest) * sizeof(float));
+  for (int i = 1; i <= started; i++) th[i - 1].join();
 }
 
 struct Builder {

@@ -118,6 +118,11 @@ __global__ __launch_bounds__(256) void rope_store_kernel(const float *__restrict
   const int r = blockIdx.x;
   const int b = r / T;
   const int pos = lens ? lens[r] - 1 : pos0 + (r - b * T);
+  if (pos < 0) {  // an empty sequence (lens[r] == 0): nothing to rotate or store, its q row is zero
+    if (q_out != nullptr)
+      for (int p = threadIdx.x; p < n_q * D; p += 256) q_out[(size_t)r * n_q * D + p] = 0.f;
+    return;
+  }
   const int half = D >> 1;
   const int q_dim = n_q * D, kv_dim = n_kv * D;
   const float *row = qkv + (size_t)r * (q_dim + 2 * kv_dim);

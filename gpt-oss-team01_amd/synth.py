@@ -42,14 +42,18 @@ def gptoss20b_config(max_seq_len: int = 1024) -> Config:
                   rope_scaling_factor=32.0, sliding_window=128, swiglu_limit=7.0)
 
 
-def random_tensors(c: Config, seed: int, std: float = 0.02) -> dict:
-    """bf16-rounded N(0, std) for every tensor; norm scales are 1 + N(0, std)."""
+def random_tensors(c: Config, seed: int, std: float = 0.02, gate_scale: float = 1.0) -> dict:
+    """bf16-rounded N(0, std) for every tensor; norm scales are 1 + N(0, std).  gate_scale (a power
+    of two, so the values stay bf16) multiplies the router's weight and bias: wider router scores,
+    fewer near-ties between the k-th and (k+1)-th expert."""
     rng = np.random.default_rng(seed)
     out = {}
     for name, shape in tensor_shapes(c).items():
         t = rng.standard_normal(size=shape, dtype=np.float32) * np.float32(std)
         if name in ("attn_norm", "mlp_norm", "final_norm"):
             t = t + np.float32(1.0)
+        if name in ("gate_weight", "gate_bias"):
+            t = t * np.float32(gate_scale)
         out[name] = bf16_round(t)
     return out
 

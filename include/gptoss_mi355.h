@@ -130,7 +130,8 @@ size_t gptoss_moe_workspace_bytes(int B, int E, int k, int H, int I);
  * (getp-csrc/src/model.cpp:74-131): router GEMM, top-k softmax, stable grouping, grouped GEMM1
  * with the token gather folded into its operand load and clamped SwiGLU folded into its epilogue
  * (kernel.cpp:560-573,636-685,927-952), grouped GEMM2 (kernel.cpp:1061-1089) and a deterministic
- * per-token weighted combine in slot order (replaces the atomicAdd scatter, kernel.cpp:748-768).
+ * per-token weighted combine in ascending expert order, the order of the CPU loop run.cpp:642-704
+ * (replaces the atomicAdd scatter, kernel.cpp:748-768).
  * t bf16 [B,H]; out fp32 [B,H].  Needs H % 64 == 0, I % 64 == 0, k <= min(8,E), E <= 256,
  * B*k*max(H,I) < 2^31. */
 int gptoss_moe_forward(const gptoss_moe_weights *w, const void *t, int B, float *out,
@@ -272,7 +273,9 @@ int gptoss_rope_tables(const gptoss_config *cfg, int n_pos, float *host_cos, flo
 /* Split the fused qkv rows [B,(n_q+2n_kv)*D] fp32, rotate q and k of sequence b for position
  * lens[b]-1 (half-split pairs, run.cpp:480-499), write q fp32 [B,n_q,D] and store k, v as bf16 into
  * slot (lens[b]-1) % capacity of the layer's cache.  cos_t / sin_t: DEVICE copies of the
- * gptoss_rope_tables arrays covering every position used.  Replaces qkv_split_rope_fused
+ * gptoss_rope_tables arrays covering every position used.  A sequence with lens[b] == 0 is empty
+ * (as for gptoss_attn_decode): nothing is stored for it and its q row is set to zero; negative
+ * lengths are treated the same way.  Replaces qkv_split_rope_fused
  * (layer_hip_batch.cpp:686-816), with a position per sequence instead of one for the batch. */
 int gptoss_rope_kv_store(const float *qkv, float *q_out, void *kv_cache, const float *cos_t,
                          const float *sin_t, const int *lens, int B, int n_q, int n_kv, int head_dim,

@@ -1,7 +1,10 @@
 #!/usr/bin/env python3
 """Writes tests/golden/tiny_e2e.json: the greedy token ids of the tiny end-to-end configuration as
 produced by the REFERENCE's own CPU model (run.cpp, compiled into oracle/_ref by oracle/Makefile),
-plus what a test needs to rebuild the same checkpoint and prompts from seeds.
+plus what a test needs to rebuild the same checkpoint and prompts from seeds; and
+tests/golden/window_e2e.json: the same for a three-layer model whose sliding window (8) is far
+shorter than the 80 positions run, so that the reference's window mask and its even-layer rule
+(run.cpp:157-164,582-584) decide the ids.
 
 Run in the build container (the reference tree is needed):
     make -C oracle ref && python tests/golden/make_golden.py
@@ -88,5 +91,93 @@ def main():
           "distinct ids", len(set(sum(fixture["expected_ids"], []))))
 
 
+WIN_REQ, WIN_PROMPT, WIN_GEN, WIN_STD, WIN_GATE_SCALE = 4, 16, 64, 0.05, 8.0
+WIN_MAX_SEQ = WIN_PROMPT + WIN_GEN
+
+
+def window_config():
+    import dataclasses
+    return dataclasses.replace(synth.tiny_config(2048), n_layers=3, hidden_dim=128, n_attn_heads=4,
+                               n_kv_heads=2, intermediate_dim=128, vocab_size=512, sliding_window=8)
+
+
+def main_window():
+    """Second fixture: positions 0..78 of a model with window 8 on its even layers (0 and 2)."""
+    import ctypes as C
+    import dataclasses
+    # seed 57 of 1..59: the only one whose router decisions (3 layers x 4 x 79 positions, fp32 and
+    # bf16-staged CPU model alike) all keep the 4th and 5th score more than 5e-3 apart, so that a
+    # bf16 engine follows the same experts all the way and every position can be compared
+    weight_seed = int(sys.argv[2]) if len(sys.argv) > 2 else 57
+    prompt_seed = 11
+    cfg = window_config()
+    with tempfile.TemporaryDirectory() as td:
+        path = os.path.join(td, "window.bin")
+        binfmt.write_bin(path, cfg, synth.random_tensors(cfg, weight_seed, std=WIN_STD, gate_scale=WIN_GATE_SCALE))
+        prompts = synth.random_prompts(cfg, WIN_REQ, WIN_PROMPT, prompt_seed)
+        sha = hashlib.sha256(open(path, "rb").read()).hexdigest()
+        ref_out, ref_n = orc.ref_generate(path, prompts, WIN_MAX_SEQ)
+        flat = np.fromfile(path, dtype="<f4", offset=binfmt.HEADER_BYTES)
+        o_out, o_n, margins = orc.generate(cfg, flat, prompts, WIN_MAX_SEQ, want_margins=True)
+        assert np.array_equal(ref_out, o_out) and ref_n == o_n, "oracle differs from the reference"
+        # how much the window decides: the same weights without a window, and with a window that
+        # covers every position, give other ids
+        no_win, _ = orc.generate(dataclasses.replace(cfg, sliding_window=0), flat, prompts, WIN_MAX_SEQ)
+        differ = int((no_win[:, :WIN_GEN] != ref_out[:, :WIN_GEN]).sum())
+        assert differ > WIN_REQ * WIN_GEN // 4, differ
+        gaps = np.zeros((WIN_REQ, WIN_GEN), np.float32)
+        min_gap = 1e9
+        R = orc.ref()
+        h = C.c_void_p(R.ref_open(path.encode()))
+        probe = []
+        for r in range(WIN_REQ):
+            m = orc.Model(cfg, flat)
+            staged = orc.Model(cfg, flat, stage=orc.STAGE_GPU)
+            seq = list(prompts[r]) + list(ref_out[r, :WIN_GEN])
+            for pos in range(WIN_MAX_SEQ - 1):
+                lg = m.forward(int(seq[pos]), pos)
+                staged.forward(int(seq[pos]), pos)
+                min_gap = min(min_gap, m.last_router_gap(), staged.last_router_gap())
+                if r == 0:
+                    # the reference's own logits, position by position, well past the window
+                    lr = np.ctypeslib.as_array(R.ref_forward(h, int(seq[pos]), pos), shape=(cfg.vocab_size,))
+                    assert np.array_equal(lg, lr), pos
+                    if pos in (7, 8, 9, 40, 78):
+                        probe.append({"pos": pos, "argmax": int(lr.argmax()), "max": float(lr.max()),
+                                      "sum": float(lr.astype(np.float64).sum())})
+                if pos >= WIN_PROMPT - 1:
+                    assert int(lg.argmax()) == ref_out[r, pos - (WIN_PROMPT - 1)]
+                    gaps[r, pos - (WIN_PROMPT - 1)] = m.last_router_gap()
+            m.close()
+            staged.close()
+        R.ref_close(h)
+        assert min_gap > 5e-3, min_gap
+    fixture = {
+        "what": "greedy ids from the reference CPU model (run.cpp forward) of a 3-layer model run ten windows "
+                "past its sliding window of 8",
+        "config": cfg.as_dict(), "weight_seed": weight_seed, "weight_std": WIN_STD, "gate_scale": WIN_GATE_SCALE,
+        "prompt_seed": prompt_seed,
+        "weights": "bf16-rounded N(0,0.05), norm scales 1+N(0,0.05), router weight and bias x8, numpy default_rng(seed) "
+                   "in tensor file order",
+        "min_router_gap_fp32_and_staged_all_positions": float(min_gap),
+        "bin_sha256": sha, "n_req": WIN_REQ, "n_prompt": WIN_PROMPT, "max_seq_len": WIN_MAX_SEQ,
+        "prompts": prompts.tolist(),
+        "expected_ids": [row[:WIN_GEN].tolist() for row in ref_out],
+        "terminator_index": WIN_GEN, "n_generated": ref_n,
+        "ids_that_differ_without_the_window": differ,
+        "min_logit_margin": float(margins[:, :WIN_GEN].min()),
+        "logit_margins": [[round(float(x), 6) for x in row[:WIN_GEN]] for row in margins],
+        "router_gaps": [[round(float(x), 6) for x in row] for row in gaps],
+        "logits_req0": probe,
+    }
+    with open(os.path.join(ROOT, "tests", "golden", "window_e2e.json"), "w") as f:
+        json.dump(fixture, f, indent=1)
+    clear = (np.asarray(fixture["logit_margins"]) > 5e-3) & (gaps > 3e-3)
+    print("wrote tests/golden/window_e2e.json; min margin", fixture["min_logit_margin"],
+          "ids that differ without the window", differ, "of", WIN_REQ * WIN_GEN,
+          "clear positions", int(clear.sum()))
+
+
 if __name__ == "__main__":
     main()
+    main_window()

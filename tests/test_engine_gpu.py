@@ -499,3 +499,89 @@ def test_prefill_and_ragged_step_edge_cases(ops, tiny):
     with pytest.raises(lib.GptossError):
         c.generate(prompts[:2, :4], 12, max_len=[8, 8])              # limits need the continuous schedule
     c.close()
+
+
+# ------------------------------------------------------------------ ten windows past the window
+WINDOW_GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "window_e2e.json")
+
+
+@pytest.fixture(scope="module")
+def windowed(synth, binfmt):
+    fx = json.load(open(WINDOW_GOLDEN))
+    cfg = binfmt.Config(**fx["config"])
+    T = synth.random_tensors(cfg, fx["weight_seed"], std=fx["weight_std"], gate_scale=fx["gate_scale"])
+    flat = np.concatenate([np.asarray(T[n], np.float32).ravel() for n in binfmt.tensor_shapes(cfg)])
+    return fx, cfg, flat
+
+
+def test_precise_engine_reproduces_the_reference_ids_past_the_window(ops, windowed):
+    """tests/golden/window_e2e.json holds what the reference's own CPU model generated for a 3-layer
+    model with a sliding window of 8 over 79 positions; 248 of the 256 ids change without the
+    window, so its mask (`pos - t >= window`) and the even-layer rule (run.cpp:157-164,582-584)
+    decide them.  The fp32-faithful engine must reproduce every id."""
+    fx, cfg, flat = windowed
+    prompts = np.asarray(fx["prompts"], np.int32)
+    gold = np.asarray(fx["expected_ids"], np.int32)
+    eng = ops.Engine(cfg, flat, max_batch=fx["n_req"], max_seq=fx["max_seq_len"], precise=True)
+    out, n = eng.generate(prompts, fx["max_seq_len"])
+    eng.close()
+    assert n == fx["n_generated"]
+    assert (out[:, fx["terminator_index"]] == -1).all()
+    assert np.array_equal(out[:, :gold.shape[1]], gold)
+
+
+def test_engine_past_the_window_matches_the_reference_ids_where_margin_is_clear(ops, orc, windowed):
+    """The same fixture through the production (bf16-staged, MFMA) engine, teacher-forced with the
+    reference's ids: lock-step steps through a 64-slot ring that holds the window of 8 (masked
+    blocks; the ring wraps at position 64), and the prompt pass over the first 70 positions (longer
+    than the ring: the linear K/V copy) followed by steps.  The fixture's weights were picked so that
+    no router decision of the fp32 or of the bf16-staged CPU model comes closer than 5e-3, so the
+    engine follows the same experts throughout and EVERY position is compared: logits within the
+    bf16 bound of the staged CPU model, and the reference's id wherever its top-1 margin exceeds
+    that bound on the logits (0.06 = 2e-2 of a logit scale of 2-3)."""
+    fx, cfg, flat = windowed
+    prompts = np.asarray(fx["prompts"], np.int32)
+    gold = np.asarray(fx["expected_ids"], np.int32)
+    margins = np.asarray(fx["logit_margins"], np.float32)
+    n_req, n_prompt = prompts.shape
+    seqs = np.concatenate([prompts, gold], axis=1)
+    assert fx["min_router_gap_fp32_and_staged_all_positions"] > 5e-3
+    clear = margins > 0.06
+    assert clear.mean() > 0.8
+    last = fx["max_seq_len"] - 1
+
+    def check(pred, what):
+        bad = np.argwhere((pred != gold) & clear & (pred >= 0))
+        assert len(bad) == 0, (what, [(int(r), int(i), float(margins[r, i])) for r, i in bad])
+
+    # lock step
+    eng = ops.Engine(cfg, flat, max_batch=n_req, max_seq=fx["max_seq_len"], keep_logits=True)
+    cpu = [orc.Model(cfg, flat, stage=orc.STAGE_GPU) for _ in range(n_req)]
+    want = np.zeros((last, n_req, cfg.vocab_size), np.float32)
+    pred = np.full_like(gold, -1)
+    worst = 0.0
+    for pos in range(last):
+        nxt = eng.step(seqs[:, pos], pos)
+        got = eng.last_logits(n_req)
+        for r in range(n_req):
+            want[pos, r] = cpu[r].forward(int(seqs[r, pos]), pos)
+            worst = max(worst, rel_errors(got[r], want[pos, r])[0])
+        if pos >= n_prompt - 1:
+            pred[:, pos - (n_prompt - 1)] = nxt
+    eng.close()
+    assert worst <= 2e-2, worst
+    check(pred, "lock step")
+    # prompt pass over 70 positions (the window layers' ring has 64 slots), then steps
+    T = 70
+    eng = ops.Engine(cfg, flat, max_batch=n_req, max_seq=fx["max_seq_len"], keep_logits=True)
+    pred = np.full_like(gold, -1)
+    pred[:, T - n_prompt] = eng.prefill(seqs[:, :T])
+    worst_pf = rel_errors(eng.last_logits(n_req), want[T - 1])[0]
+    for pos in range(T, last):
+        pred[:, pos - (n_prompt - 1)] = eng.step(seqs[:, pos], pos)
+        worst_pf = max(worst_pf, rel_errors(eng.last_logits(n_req), want[pos])[0])
+    eng.close()
+    assert worst_pf <= 2e-2, worst_pf
+    check(pred, "prompt pass")
+    print("window fixture: ids compared", int(clear.sum()), "of", clear.size, "; worst max-rel vs the staged CPU model:",
+          "lock step", worst, "prompt pass + steps", worst_pf)

@@ -266,20 +266,95 @@ def test_oracle_forward_bit_identical_to_reference_cpu(tiny, orc):
 
 
 def test_sliding_window_layers_are_the_even_ones(orc, synth):
-    """Past the window, even layers stop seeing old positions: with window 4 the logits at
-    position 6 must differ from a window-free run, and must not if the window covers everything."""
+    """run.cpp:582-584 masks positions `pos - t >= window` on layers with `l % 2 == 0`.  Two-layer
+    model, window 4, 7 positions.  With the output projection of layer 1 zeroed only layer 0's
+    attention reaches the logits: they must change with the window (layer 0 is windowed).  With the
+    output projection of layer 0 zeroed instead only layer 1's attention does: they must not change
+    (layer 1 sees every position).  An oracle that windowed the odd layers fails both halves."""
     import dataclasses
     base = dataclasses.replace(synth.tiny_config(16), n_layers=2, vocab_size=64, sliding_window=4)
     from conftest import load_pkg
     binfmt = load_pkg("binfmt")
-    T = synth.random_tensors(base, 3, std=0.2)
-    flat = np.concatenate([np.asarray(T[n], np.float32).ravel() for n in binfmt.tensor_shapes(base)])
-    def run(cfg):
+
+    def run(cfg, mute_layer=None, n_pos=7):
+        T = synth.random_tensors(base, 3, std=0.2)
+        if mute_layer is not None:
+            T["out_weight"][mute_layer] = 0
+            T["out_bias"][mute_layer] = 0
+        flat = np.concatenate([np.asarray(T[n], np.float32).ravel() for n in binfmt.tensor_shapes(base)])
         m = orc.Model(cfg, flat)
-        for pos in range(7):
+        for pos in range(n_pos):
             lg = m.forward(pos + 1, pos)
         return lg
+
+    no_window = dataclasses.replace(base, sliding_window=0)
     a = run(base)
-    b = run(dataclasses.replace(base, sliding_window=0))
+    b = run(no_window)
     c = run(dataclasses.replace(base, sliding_window=16))
     assert not np.allclose(a, b) and np.array_equal(b, c)
+    assert not np.allclose(run(base, mute_layer=1), run(no_window, mute_layer=1))      # layer 0: windowed
+    assert np.array_equal(run(base, mute_layer=0), run(no_window, mute_layer=0))       # layer 1: not
+    # the mask is `pos - t >= window`: at position window-1 nothing is masked yet, at position window
+    # exactly one position is
+    assert np.array_equal(run(base, 1, n_pos=4), run(no_window, 1, n_pos=4))
+    assert not np.array_equal(run(base, 1, n_pos=5), run(no_window, 1, n_pos=5))
+
+
+WINDOW_GOLDEN = os.path.join(HERE, "golden", "window_e2e.json")
+
+
+@pytest.fixture(scope="module")
+def windowed(synth, binfmt, tmp_path_factory):
+    fx = json.load(open(WINDOW_GOLDEN))
+    cfg = binfmt.Config(**fx["config"])
+    path = str(tmp_path_factory.mktemp("window") / "window.bin")
+    binfmt.write_bin(path, cfg, synth.random_tensors(cfg, fx["weight_seed"], std=fx["weight_std"], gate_scale=fx["gate_scale"]))
+    assert hashlib.sha256(open(path, "rb").read()).hexdigest() == fx["bin_sha256"]
+    return fx, cfg, path
+
+
+def test_oracle_matches_the_reference_ids_past_the_window(windowed, orc):
+    """tests/golden/window_e2e.json: ids and logit probes the reference's own CPU model produced for
+    a 3-layer model with window 8 over 79 positions (248 of the 256 ids change when the window is
+    taken away, so the mask and the even-layer rule decide them)."""
+    fx, cfg, path = windowed
+    flat = np.fromfile(path, dtype="<f4", offset=60)
+    prompts = np.asarray(fx["prompts"], np.int32)
+    out, n = orc.generate(cfg, flat, prompts, fx["max_seq_len"])
+    gold = np.asarray(fx["expected_ids"], np.int32)
+    np.testing.assert_array_equal(out[:, :gold.shape[1]], gold)
+    assert (out[:, fx["terminator_index"]] == -1).all() and n == fx["n_generated"]
+    m = orc.Model(cfg, flat)
+    seq = list(prompts[0]) + list(gold[0])
+    probes = {p["pos"]: p for p in fx["logits_req0"]}
+    for pos in range(fx["max_seq_len"] - 1):
+        lg = m.forward(int(seq[pos]), pos)
+        if pos in probes:
+            assert int(lg.argmax()) == probes[pos]["argmax"]
+            assert float(lg.max()) == probes[pos]["max"]
+            np.testing.assert_allclose(lg.astype(np.float64).sum(), probes[pos]["sum"], rtol=1e-9)
+
+
+def test_oracle_forward_bit_identical_to_reference_cpu_past_the_window(orc, synth, binfmt, tmp_path):
+    """The reference's own compiled forward() against the oracle, logits bit for bit, on models that
+    run well past their sliding window (run.cpp:157-164,582-584): windows 4..8, 3 and 4 layers,
+    24 positions."""
+    if not orc.have_ref():
+        pytest.skip("oracle/_ref not built (reference tree absent)")
+    import dataclasses
+    R = orc.ref()
+    rng = np.random.default_rng(12)
+    for window, layers in ((4, 3), (6, 4), (8, 3)):
+        cfg = dataclasses.replace(synth.tiny_config(2048), n_layers=layers, hidden_dim=128, n_attn_heads=4,
+                                  n_kv_heads=2, intermediate_dim=64, vocab_size=256, sliding_window=window)
+        path = str(tmp_path / f"w{window}.bin")
+        binfmt.write_bin(path, cfg, synth.random_tensors(cfg, 40 + window, std=0.08))
+        flat = np.fromfile(path, dtype="<f4", offset=60)
+        h = C.c_void_p(R.ref_open(path.encode()))
+        m = orc.Model(cfg, flat)
+        for pos in range(24):
+            tok = int(rng.integers(cfg.vocab_size))
+            lr = np.ctypeslib.as_array(R.ref_forward(h, tok, pos), shape=(cfg.vocab_size,)).copy()
+            np.testing.assert_array_equal(m.forward(tok, pos), lr, err_msg=f"window {window} pos {pos}")
+        R.ref_close(h)
+        m.close()

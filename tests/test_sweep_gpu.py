@@ -84,11 +84,95 @@ def test_attn_random_shapes(ops, orc):
     print("random attention shapes: worst max-rel / mean-rel", worst)
 
 
+#: a router decision closer than this (k-th against (k+1)-th score, relative to the score scale of
+#: these models) may fall the other way under a different summation order
+ROUTER_NEAR_TIE = 3e-3
+
+
+def _engine_case(ops, orc, binfmt, D, nq, nkv, H, E, k, I, L, V, win, B, T, seed, tok_cols):
+    """One model configuration through lock-step steps, the prompt pass and one ragged step.
+    Returns the worst max-rel of the lock-step rows against the staged CPU model and the rows of
+    the prompt pass that a router near-tie excused."""
+    cfg = binfmt.Config(vocab_size=V, hidden_dim=H, n_experts=E, experts_per_token=k, intermediate_dim=I,
+                        n_layers=L, head_dim=D, n_attn_heads=nq, n_kv_heads=nkv, seq_len=2048,
+                        initial_context_length=4096, rope_theta=150000.0, rope_scaling_factor=32.0,
+                        sliding_window=win, swiglu_limit=7.0)
+    g = np.random.default_rng(seed)
+    flat = np.empty(binfmt.n_weight_floats(cfg), np.float32)
+    off = 0
+    for name, shape in binfmt.tensor_shapes(cfg).items():
+        m = int(np.prod(shape))
+        x = g.standard_normal(m).astype(np.float32) * 0.05
+        if name in ("attn_norm", "mlp_norm", "final_norm"):
+            x = x * 0.4 + 1.0
+        flat[off:off + m] = torch.from_numpy(x).to(torch.bfloat16).float().numpy()
+        off += m
+    toks = g.integers(0, V, size=(B, tok_cols)).astype(np.int32)
+    a = ops.Engine(cfg, flat, max_batch=B, max_seq=128, keep_logits=True)
+    b = ops.Engine(cfg, flat, max_batch=B, max_seq=128, keep_logits=True)
+    rows = sorted({0, B // 2, B - 1})
+    cpu = {r: orc.Model(cfg, flat, stage=orc.STAGE_GPU) for r in rows}
+    live = set(rows)
+    worst = 0.0
+    for pos in range(T):
+        ids = a.step(toks[:, pos], pos)
+        got = a.last_logits(B)
+        assert np.array_equal(ids, got.argmax(axis=1)), (pos, cfg)
+        for r in rows:
+            want = cpu[r].forward(int(toks[r, pos]), pos)
+            if cpu[r].last_router_gap() < 1.5e-2:
+                live.discard(r)
+            if r in live:
+                mx, _ = rel_errors(got[r], want)
+                worst = max(worst, mx)
+                assert mx <= 2e-2, (pos, r, mx, cfg)
+    b.prefill(toks[:, :T])
+    lb = b.last_logits(B)
+    excused = []
+    if T <= win:
+        assert np.array_equal(lb, got), ("prompt pass differs from lock step", cfg)
+    else:
+        # A ring has wrapped: the prompt pass sums the window in position order, the lock-step
+        # step in slot order, so the two differ by fp32 summation order and, through the bf16
+        # roundings, by a last bit here and there.  Every row must stay within the bf16 bound
+        # unless, on the positions where the orders differ, the staged CPU model shows a router
+        # decision of that row close enough to fall the other way.
+        per = np.abs(lb - got).max(axis=1) / np.abs(got).max(axis=1)
+        assert np.median(per) <= 5e-3, (per, cfg)
+        for r in np.nonzero(per > TOL_MAX)[0]:
+            m = orc.Model(cfg, flat, stage=orc.STAGE_GPU)
+            gaps = []
+            for pos in range(T):
+                m.forward(int(toks[r, pos]), pos)
+                gaps.append(m.last_router_gap())
+            m.close()
+            tie = min(gaps[win:])
+            assert tie < ROUTER_NEAR_TIE, ("prompt pass row beyond bf16 tolerance without a router near-tie",
+                                           int(r), float(per[r]), tie, cfg)
+            excused.append((int(r), float(per[r]), float(tie), win + int(np.argmin(gaps[win:]))))
+        assert len(excused) <= max(1, B // 8), (excused, cfg)
+    posv = np.array([T - (i % 2) for i in range(B)], np.int32)   # every other row repeats its last position
+    a.step_ragged(np.array([toks[i, posv[i]] for i in range(B)], np.int32), posv)
+    lr = a.last_logits(B)
+    for r in rows:
+        if r in live and posv[r] == T:
+            want = cpu[r].forward(int(toks[r, T]), T)
+            if cpu[r].last_router_gap() >= 1.5e-2:
+                mx, _ = rel_errors(lr[r], want)
+                assert mx <= 2e-2, ("ragged", r, mx, cfg)
+    a.close()
+    b.close()
+    for m in cpu.values():
+        m.close()
+    return worst, excused
+
+
 def test_engine_random_configs(ops, orc, binfmt):
     """Lock-step steps against the CPU model that rounds where the GPU dataflow rounds (rows are
     dropped once a router decision comes closer than 1.5e-2: the two may then pick different
     experts), the prompt pass against the lock-step steps (bit for bit while no sliding-window ring
-    has wrapped), and one step with per-sequence positions."""
+    has wrapped; per row within the bf16 bound after, router near-ties excepted), and one step
+    with per-sequence positions."""
     rng = np.random.default_rng(20242)
     done = 0
     worst = 0.0
@@ -108,57 +192,20 @@ def test_engine_random_configs(ops, orc, binfmt):
         T = int(rng.choice([3, 9, 70 if win == 64 else 20]))
         if ((nq + 2 * nkv) * D) % 64 or (nq * D) % 64:
             continue                                         # the engine wants these multiples of 64
-        cfg = binfmt.Config(vocab_size=V, hidden_dim=H, n_experts=E, experts_per_token=k, intermediate_dim=I,
-                            n_layers=L, head_dim=D, n_attn_heads=nq, n_kv_heads=nkv, seq_len=2048,
-                            initial_context_length=4096, rope_theta=150000.0, rope_scaling_factor=32.0,
-                            sliding_window=win, swiglu_limit=7.0)
-        g = np.random.default_rng(seed)
-        flat = np.empty(binfmt.n_weight_floats(cfg), np.float32)
-        off = 0
-        for name, shape in binfmt.tensor_shapes(cfg).items():
-            m = int(np.prod(shape))
-            x = g.standard_normal(m).astype(np.float32) * 0.05
-            if name in ("attn_norm", "mlp_norm", "final_norm"):
-                x = x * 0.4 + 1.0
-            flat[off:off + m] = torch.from_numpy(x).to(torch.bfloat16).float().numpy()
-            off += m
-        toks = g.integers(0, V, size=(B, T + 1)).astype(np.int32)
-        a = ops.Engine(cfg, flat, max_batch=B, max_seq=128, keep_logits=True)
-        b = ops.Engine(cfg, flat, max_batch=B, max_seq=128, keep_logits=True)
-        rows = sorted({0, B // 2, B - 1})
-        cpu = {r: orc.Model(cfg, flat, stage=orc.STAGE_GPU) for r in rows}
-        live = set(rows)
-        for pos in range(T):
-            ids = a.step(toks[:, pos], pos)
-            got = a.last_logits(B)
-            assert np.array_equal(ids, got.argmax(axis=1)), (done, pos)
-            for r in rows:
-                want = cpu[r].forward(int(toks[r, pos]), pos)
-                if cpu[r].last_router_gap() < 1.5e-2:
-                    live.discard(r)
-                if r in live:
-                    mx, _ = rel_errors(got[r], want)
-                    worst = max(worst, mx)
-                    assert mx <= 2e-2, (done, pos, r, mx, cfg)
-        b.prefill(toks[:, :T])
-        lb = b.last_logits(B)
-        if T <= win:
-            assert np.array_equal(lb, got), (done, "prompt pass differs from lock step", cfg)
-        else:
-            per = np.abs(lb - got).max(axis=1) / np.abs(got).max(axis=1)
-            assert np.median(per) <= 5e-3, (done, per, cfg)
-        posv = np.array([T - (i % 2) for i in range(B)], np.int32)   # every other row repeats its last position
-        a.step_ragged(np.array([toks[i, posv[i]] for i in range(B)], np.int32), posv)
-        lr = a.last_logits(B)
-        for r in rows:
-            if r in live and posv[r] == T:
-                want = cpu[r].forward(int(toks[r, T]), T)
-                if cpu[r].last_router_gap() >= 1.5e-2:
-                    mx, _ = rel_errors(lr[r], want)
-                    assert mx <= 2e-2, (done, "ragged", r, mx, cfg)
-        a.close()
-        b.close()
-        for m in cpu.values():
-            m.close()
+        w, _ = _engine_case(ops, orc, binfmt, D, nq, nkv, H, E, k, I, L, V, win, B, T, seed, T + 1)
+        worst = max(worst, w)
         done += 1
     print("random engine configurations: worst max-rel against the staged CPU model", worst)
+
+
+def test_prompt_pass_past_the_window_differs_from_lock_step_only_at_router_near_ties(ops, orc, binfmt):
+    """A case a long run of the generator above turned up: 33 sequences, 70-token prompt, window 64,
+    top-2 of 32 experts.  One row's logits after the prompt pass differ from the lock-step ones by
+    most of their scale.  The staged CPU model puts that row's 2nd and 3rd router scores at
+    position 69 only 3.1e-4 apart (row 19; the next closest decision at that position in the whole
+    batch is ten times wider), so the two summation orders of the wrapped window pick different
+    experts there; every other row agrees within the bf16 bound."""
+    _, excused = _engine_case(ops, orc, binfmt, D=32, nq=2, nkv=2, H=320, E=32, k=2, I=128, L=2, V=512, win=64,
+                              B=33, T=70, seed=355231429, tok_cols=72)
+    print("rows excused by a router near-tie (row, max-rel, gap, position):", excused)
+    assert [e[0] for e in excused] in ([19], []), excused
