@@ -68,6 +68,9 @@ def parse():
     ap.add_argument("--no-zipf", action="store_true",
                     help="skip the skewed-routing figure of the headline layer (profile runs: every "
                          "launch of the roofline kernel is then the headline workload)")
+    ap.add_argument("--mfma-rates", action="store_true",
+                    help="only measure the register-fed issue rate of the bf16 and the scaled f8f6f4 MFMA "
+                         "(gptoss_diag_mfma_rate) and print one JSON line of its own")
     ap.add_argument("--no-sched", action="store_true", help="skip the scheduler leg of the end-to-end figure")
     return ap.parse_args()
 
@@ -296,6 +299,66 @@ def bench_attn(ops, torch, steps, warmup):
         res[name] = {"us": round(ms * 1e3, 1), "kv_mb": round(kv_bytes / 1e6, 1),
                      "gbs": round(kv_bytes / ms / 1e6, 1),
                      "hbm_frac": round(kv_bytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
+    del caches, attn
+    res["engine_shapes_position_383"] = bench_attn_engine_shapes(ops, torch, steps, warmup)
+    res["prompt_attention"] = bench_attn_prompt(ops, torch)
+    return res
+
+
+def bench_attn_engine_shapes(ops, torch, steps, warmup):
+    """The two attention calls of a layer pair of the whole-model decode step at its last position
+    (configs[3]: 1024 sequences, position 383): a full layer (384 cached positions, one length for
+    the batch) and a sliding-window layer (128-slot ring that has wrapped, every slot active)."""
+    B, n_q, n_kv, D, pos = 1024, 64, 8, 64, 383
+    q = torch.randn(B, n_q, D, device="cuda")
+    sinks = torch.randn(n_q, device="cuda")
+    out = torch.empty(B, n_q, D, dtype=torch.bfloat16, device="cuda")
+    res = {}
+    for name, cap, window in (("full_384", 384, 0), ("window_ring_128", 128, 128)):
+        caches = []
+        for _ in range(2):
+            c = ops.KVCache(B, n_kv, D, cap)
+            c.kv.normal_()
+            caches.append(c)
+        attn = ops.AttnDecode(B, n_q, n_kv, D, pos + 1)
+        for i in range(warmup):
+            attn.forward(q, caches[i % 2], None, sinks, window=window, out=out, max_len=pos + 1)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(steps):
+            attn.forward(q, caches[i % 2], None, sinks, window=window, out=out, max_len=pos + 1)
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) * 1e3 / steps
+        kv_bytes = B * min(pos + 1, cap) * n_kv * D * 2 * 2
+        res[name] = {"us": round(ms * 1e3, 1), "kv_mb": round(kv_bytes / 1e6, 1),
+                     "gbs": round(kv_bytes / ms / 1e6, 1),
+                     "hbm_frac": round(kv_bytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
+        del caches, attn
+    return res
+
+
+def bench_attn_prompt(ops, torch):
+    """Prompt attention of one layer for 8192 rows: 64 prompts of 128 positions against 8 prompts of
+    1024 positions (the reference's cap), full and with the 128-position window."""
+    n_q, n_kv, D = 64, 8, 64
+    res = {}
+    for B, T in ((64, 128), (8, 1024)):
+        q = torch.randn(B, T, n_q, D, device="cuda")
+        cache = ops.KVCache(B, n_kv, D, T)
+        cache.kv.normal_()
+        sinks = torch.randn(n_q, device="cuda")
+        pre = ops.AttnPrefill(B, T, n_q, n_kv, D, T)
+        for name, window in (("full", 0), ("window128", 128)):
+            for _ in range(3):
+                pre.forward(q, cache, pos0=0, sinks=sinks, window=window)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(10):
+                pre.forward(q, cache, pos0=0, sinks=sinks, window=window)
+            e1.record()
+            torch.cuda.synchronize()
+            res[f"{B}x{T}_{name}_us"] = round(e0.elapsed_time(e1) * 100, 1)
+        del q, cache, pre
     return res
 
 
@@ -465,6 +528,28 @@ def bench_loader(ops, torch):
             "what": "fp32 host payload (20B dimensions, 2 blocks) -> packed bf16 device weights, PCIe included"}
 
 
+def bench_mfma_rates(torch):
+    """Register-fed rate of the matrix instructions (no loads, no LDS): 256 workgroups of 8 waves."""
+    import ctypes as C
+    L = importlib.import_module("gpt-oss-team01_amd.lib")
+    lib = L.load()
+    sink = torch.zeros(16, dtype=torch.float32, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    names = ("bf16_32x32x16", "scaled_fp8_x_fp4_32x32x64", "scaled_fp4_x_fp4_32x32x64", "scaled_fp8_x_fp8_32x32x64")
+    out = {}
+    for kind, name in enumerate(names):
+        flop = C.c_double(0)
+        for timed in (False, True):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            L.check(lib.gptoss_diag_mfma_rate(kind, 256, 20000, sink.data_ptr(), C.byref(flop), stream))
+            e1.record()
+            torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1)
+        out[name] = {"ms": round(ms, 3), "tflops": round(flop.value / ms / 1e9, 1)}
+    return out
+
+
 def main():
     args = parse()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -477,6 +562,10 @@ def main():
         sys.exit(3)
     importlib.import_module("gpt-oss-team01_amd.lib").load()
     ops = importlib.import_module("gpt-oss-team01_amd.ops")
+    if args.mfma_rates:
+        print(json.dumps({"what": "register-fed MFMA issue rates, 256 workgroups x 8 waves x 4 accumulators",
+                          "rates": bench_mfma_rates(torch)}))
+        return
 
     # a plain device copy of known size (2 x 1 GiB moved), so counter runs of this same command can
     # be scaled by what the counters read for it

@@ -27,6 +27,8 @@
 //   * several query rows may share one sequence's cache (rows_per_seq), each with its own length:
 //     the T positions of a prompt are T such rows, which is all the prompt-pass attention is; two
 //     consecutive rows of a sequence then share a wave (8 heads each in the 16 operand columns).
+#include <stdlib.h>
+
 #include <algorithm>
 #include <mutex>
 #include <type_traits>
@@ -526,6 +528,223 @@ __global__ __launch_bounds__(256) void attn_reduce_kernel(AttnParams p) {
   *reinterpret_cast<u32x2 *>(p.out + ((size_t)b * p.n_q + hq) * D + d4) = pk;
 }
 
+// Prompt attention for many positions of one sequence: a workgroup of 8 waves serves 16
+// consecutive query rows of one (sequence, kv head), two rows per wave as in the PAIR form above,
+// and walks the K/V blocks any of them needs ONCE: every block goes from global memory into LDS
+// (two buffers, one barrier per block) and the eight waves take their operands from there.  The
+// pair form reads a sequence's cache once per row pair, which is quadratic traffic for long
+// prompts; here it is read once per 16 rows, and the pass is bound by the matrix instructions.
+// Every row sees the arithmetic of the one-wave kernel over its own blocks in ascending order (a
+// block outside a row's range is a no-op for its columns), so rows of up to ATT_CHUNK positions
+// equal the decode call bit for bit; longer rows are summed in one pass instead of chunk by
+// chunk.  Needs slot == position (no wrapped ring) and at most 8 query heads per kv head.
+constexpr int TILE_WAVES = 8;
+constexpr int TILE_ROWS = 2 * TILE_WAVES;
+
+template <int D>
+__global__ __launch_bounds__(TILE_WAVES * 64, 4) void attn_prefill_tile_kernel(AttnParams p) {
+  constexpr int KS = D / 32;
+  constexpr int DB = D / 16;
+  constexpr int BLOCK_BYTES = 2 * KV_BLOCK * D * 2;        // K rows then V fragments of 64 slots
+  constexpr int K_BYTES = KV_BLOCK * D * 2;
+  constexpr int CHUNKS = BLOCK_BYTES / 16;                   // 16-byte pieces per block
+  constexpr int PASSES = CHUNKS / (TILE_WAVES * 64);         // pieces per thread
+  constexpr int ROW_CHUNKS = D / 8;                          // 16-byte pieces per K row
+  static_assert(PASSES >= 1 && CHUNKS % (TILE_WAVES * 64) == 0, "block size against workgroup size");
+  __shared__ __attribute__((aligned(16))) unsigned char lds[2][BLOCK_BYTES];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int T = p.rows_per_seq;
+  const int groups = (T + TILE_ROWS - 1) / TILE_ROWS;
+  const int n_seq = p.B / T;
+  // late row groups first: they walk the most blocks
+  const int g = blockIdx.x % p.n_kv;
+  const int rest = blockIdx.x / p.n_kv;
+  const int seq = rest % n_seq;
+  const int rg = groups - 1 - rest / n_seq;
+  const int t0 = rg * TILE_ROWS;                             // first row of the group within the sequence
+  const int t_last = min(T, t0 + TILE_ROWS) - 1;
+  // active positions of row t: [lo(t), hi(t)), hi(t) = len_base + t
+  auto row_hi = [&](int t) { return min(p.len_base + t, p.max_len); };
+  auto row_lo = [&](int t) { return p.window > 0 ? max(0, row_hi(t) - p.window) : 0; };
+  const int blk_begin = row_lo(t0) & ~(ATT_BLOCK - 1);
+  const int blk_end = row_hi(t_last);
+  // this wave's two rows
+  const int tw = t0 + 2 * wave;
+  const bool have0 = tw < T, two = tw + 1 < T;
+  const int lo0 = have0 ? row_lo(tw) : 0, hi0 = have0 ? row_hi(tw) : 0;
+  const int lo1 = two ? row_lo(tw + 1) : 0, hi1 = two ? row_hi(tw + 1) : 0;
+  const int b = seq * T + (have0 ? tw : 0);                  // query row of the first of them
+  const int n = lane & 15, c = lane >> 4;
+  const int G = p.G;
+  const bool second = n >= 8;
+  const int hn = n & 7;
+  const bool col_live = have0 && hn < G && (!second || two);
+  const int bn = (second && two) ? b + 1 : b;
+  const int head = g * G + min(hn, G - 1);
+  const float sink_logit = p.sinks ? p.sinks[head] : -INFINITY;
+
+  const unsigned char *plane = reinterpret_cast<const unsigned char *>(p.kv + kv_block_off(seq, g, p.n_kv, p.cap, D, 0));
+  // the workgroup's copy of a block: piece i of thread t is bytes (i * 512 + t) * 16; a K piece is
+  // chunk j of row r and lands at chunk position j ^ swz(r) of its row, so that the 16 lanes of a
+  // fragment read (16 rows, one chunk) hit 16 different 16-byte slots modulo 256 bytes
+  auto swz = [](int r) { return D == 64 ? ((r >> 1) & 7) : ((r >> 2) & 3); };
+  u32x4 stage[PASSES];
+  auto load_block = [&](int blk) {
+    const unsigned char *src = plane + (size_t)(blk >> 6) * BLOCK_BYTES;
+#pragma unroll
+    for (int i = 0; i < PASSES; i++)
+      stage[i] = *reinterpret_cast<const u32x4 *>(src + (size_t)(i * TILE_WAVES * 64 + tid) * 16);
+  };
+  auto store_block = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < PASSES; i++) {
+      const int piece = i * TILE_WAVES * 64 + tid;
+      int dst = piece * 16;
+      if (piece * 16 < K_BYTES) {
+        const int r = piece / ROW_CHUNKS, j = piece % ROW_CHUNKS;
+        dst = r * (D * 2) + ((j ^ swz(r)) << 4);
+      }
+      *reinterpret_cast<u32x4 *>(&lds[buf][dst]) = stage[i];
+    }
+  };
+  if (blk_end > blk_begin) load_block(blk_begin);
+
+  bf16x8 qh[KS], ql[KS];
+  {
+    const float *qp = p.q + ((size_t)bn * p.n_q + head) * D + c * KS * 8;
+#pragma unroll
+    for (int s = 0; s < KS; s++) {
+      uint32_t h[4], l[4];
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        float x0 = col_live ? qp[s * 8 + 2 * j] : 0.f, x1 = col_live ? qp[s * 8 + 2 * j + 1] : 0.f;
+        bf16_t h0 = f32_to_bf16(x0), h1 = f32_to_bf16(x1);
+        h[j] = (uint32_t)h0 | ((uint32_t)h1 << 16);
+        l[j] = pack_bf16x2(x0 - bf16_to_f32(h0), x1 - bf16_to_f32(h1));
+      }
+      qh[s] = as_bf16x8(u32x4{h[0], h[1], h[2], h[3]});
+      ql[s] = as_bf16x8(u32x4{l[0], l[1], l[2], l[3]});
+    }
+  }
+  f32x4 o[DB];
+#pragma unroll
+  for (int db = 0; db < DB; db++) o[db] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m_run = NEG_BIG, l_run = 0.f;
+  const int lane_lo = second ? lo1 : lo0, lane_hi = second ? hi1 : hi0;
+
+  // one 64-slot block from LDS buffer `buf`: the arithmetic of the one-wave kernel's block step
+  auto process = [&](int blk, int buf, auto edge_sel) {
+    constexpr bool EDGE = decltype(edge_sel)::value;
+    const unsigned char *kb = lds[buf];
+    const unsigned char *vb = lds[buf] + K_BYTES;
+    f32x4 s4[4];
+#pragma unroll
+    for (int tb = 0; tb < 4; tb++) {
+      f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+      const int r = tb * 16 + n;
+#pragma unroll
+      for (int s = 0; s < KS; s++) {
+        const bf16x8 kf = as_bf16x8(*reinterpret_cast<const u32x4 *>(kb + r * (D * 2) + (((c * KS + s) ^ swz(r)) << 4)));
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qh[s], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, ql[s], acc, 0, 0, 0);
+      }
+      s4[tb] = acc;
+    }
+    float bmax = NEG_BIG;
+#pragma unroll
+    for (int tb = 0; tb < 4; tb++)
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        float v = s4[tb][i] * p.scale_log2e;
+        asm volatile("" : "+v"(v));   // a rounded product of its own, as in the one-wave kernel
+        if (EDGE) {
+          const int slot = blk + tb * 16 + c * 4 + i;
+          v = (slot >= lane_lo && slot < lane_hi) ? v : -INFINITY;
+        }
+        s4[tb][i] = v;
+        bmax = fmaxf(bmax, v);
+      }
+    bmax = fmaxf(bmax, __shfl_xor(bmax, 16, 64));
+    bmax = fmaxf(bmax, __shfl_xor(bmax, 32, 64));
+    const float m_new = fmaxf(m_run, bmax);
+    const float alpha = exp2f(m_run - m_new);
+    m_run = m_new;
+    float psum = 0.f;
+    bf16x8 ph[2], pl[2];
+#pragma unroll
+    for (int grp = 0; grp < 2; grp++) {
+      uint32_t h[4], l[4];
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        float p0 = exp2f(s4[grp * 2 + (j >> 1)][(j & 1) * 2] - m_new);
+        float p1 = exp2f(s4[grp * 2 + (j >> 1)][(j & 1) * 2 + 1] - m_new);
+        psum += p0 + p1;
+        uint32_t u0 = __float_as_uint(p0), u1 = __float_as_uint(p1);
+        h[j] = (u0 >> 16) | (u1 & 0xffff0000u);
+        float r0 = p0 - __uint_as_float(u0 & 0xffff0000u), r1 = p1 - __uint_as_float(u1 & 0xffff0000u);
+        l[j] = (__float_as_uint(r0) >> 16) | (__float_as_uint(r1) & 0xffff0000u);
+      }
+      ph[grp] = as_bf16x8(u32x4{h[0], h[1], h[2], h[3]});
+      pl[grp] = as_bf16x8(u32x4{l[0], l[1], l[2], l[3]});
+    }
+    l_run = l_run * alpha + psum;
+#pragma unroll
+    for (int db = 0; db < DB; db++) {
+#pragma unroll
+      for (int i = 0; i < 4; i++) o[db][i] *= alpha;
+    }
+#pragma unroll
+    for (int grp = 0; grp < 2; grp++)
+#pragma unroll
+      for (int db = 0; db < DB; db++) {
+        u32x4 vv = *reinterpret_cast<const u32x4 *>(vb + (grp * DB + db) * 1024 + lane * 16);
+        if (EDGE) {
+#pragma unroll
+          for (int w = 0; w < 4; w++) {
+            const int s_lo = blk + grp * 32 + (w >> 1) * 16 + c * 4 + (w & 1) * 2;
+            auto used = [&](int sl) { return (sl >= lo0 && sl < hi0) || (sl >= lo1 && sl < hi1); };
+            const uint32_t keep = (used(s_lo) ? 0x0000ffffu : 0u) | (used(s_lo + 1) ? 0xffff0000u : 0u);
+            vv[w] &= keep;
+          }
+        }
+        bf16x8 vf = as_bf16x8(vv);
+        o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, ph[grp], o[db], 0, 0, 0);
+        o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pl[grp], o[db], 0, 0, 0);
+      }
+  };
+
+  int buf = 0;
+  for (int blk = blk_begin; blk < blk_end; blk += ATT_BLOCK, buf ^= 1) {
+    store_block(buf);
+    __syncthreads();   // block `blk` is complete in lds[buf]; every wave is done with the other buffer's previous use
+    if (blk + ATT_BLOCK < blk_end) load_block(blk + ATT_BLOCK);
+    // the wave's rows: first block that holds an active position of either row .. their last one
+    const bool mine = (have0 && blk < hi0 && blk + ATT_BLOCK > lo0) || (two && blk < hi1 && blk + ATT_BLOCK > lo1);
+    if (mine) {
+      const bool edge = !(two && blk >= lo0 && blk + ATT_BLOCK <= hi0 && blk >= lo1 && blk + ATT_BLOCK <= hi1);
+      if (edge) process(blk, buf, std::true_type{});
+      else process(blk, buf, std::false_type{});
+    }
+  }
+
+  l_run += __shfl_xor(l_run, 16, 64);
+  l_run += __shfl_xor(l_run, 32, 64);
+  if (!col_live) return;
+  const int hq = g * G + hn;
+  const float sink2 = sink_logit * 1.4426950408889634f;
+  const float M = fmaxf(m_run, sink2);
+  const float w = exp2f(m_run - M);
+  const float denom = l_run * w + exp2f(sink2 - M);
+  const float inv = (denom > 0.f) ? w / denom : 0.f;
+  bf16_t *op = p.out + ((size_t)bn * p.n_q + hq) * D;
+#pragma unroll
+  for (int db = 0; db < DB; db++) {
+    u32x2 pk = u32x2{pack_bf16x2(o[db][0] * inv, o[db][1] * inv), pack_bf16x2(o[db][2] * inv, o[db][3] * inv)};
+    *reinterpret_cast<u32x2 *>(op + db * 16 + c * 4) = pk;
+  }
+}
+
 // Bulk cache write: rows [B, n_tok, n_kv, D] -> the block layout of common.hpp.
 __global__ __launch_bounds__(256) void kv_cache_write_kernel(bf16_t *__restrict__ kv,
                                                              const bf16_t *__restrict__ k_rows,
@@ -545,6 +764,17 @@ __global__ __launch_bounds__(256) void kv_cache_write_kernel(bf16_t *__restrict_
     kv[base + kv_k_elem(slot, d, D)] = k_rows[i];
     kv[base + kv_v_elem(slot, d, D)] = v_rows[i];
   }
+}
+
+// Positions per sequence from which a prompt pass takes the tiled kernel.  GPTOSS_ATTN_TILE_MIN_ROWS
+// overrides it (tests run both forms on the same inputs).
+static int attn_tile_min_rows() {
+  static const int v = [] {
+    const char *e = getenv("GPTOSS_ATTN_TILE_MIN_ROWS");
+    const int n = e ? atoi(e) : 0;
+    return n > 0 ? n : 32;
+  }();
+  return v;
 }
 
 struct AttnPlan {
@@ -665,6 +895,16 @@ static int attn_launch(const float *q, const void *kv_cache, const int *lens,
   // prompt passes put two consecutive rows of a sequence into one wave when the 16 operand columns
   // hold both rows' query heads and no ring can have wrapped (slot == position)
   const bool pair = rows_per_seq > 1 && B % rows_per_seq == 0 && p.G <= 8 && max_len <= capacity;
+  if (pair && rows_per_seq >= attn_tile_min_rows()) {
+    // many positions per sequence: 16 rows per workgroup share every K/V block through LDS
+    const long long wgs = (long long)(B / rows_per_seq) * n_kv * ((rows_per_seq + TILE_ROWS - 1) / TILE_ROWS);
+    GPTOSS_REQUIRE(wgs < (1ll << 31), GPTOSS_ERR_DIM, "attn_prefill: too many row groups (%lld)", wgs);
+    TraceScope ts("attn_prefill_tiles", s);
+    if (head_dim == 64) attn_prefill_tile_kernel<64><<<(int)wgs, TILE_WAVES * 64, 0, s>>>(p);
+    else attn_prefill_tile_kernel<32><<<(int)wgs, TILE_WAVES * 64, 0, s>>>(p);
+    GPTOSS_LAUNCH_CHECK("attn_prefill_tile_kernel");
+    return GPTOSS_OK;
+  }
   long long items = (long long)(pair ? (B / rows_per_seq) * ((rows_per_seq + 1) / 2) : B) * n_kv * p.max_chunks;
   int grid = (int)((items + 3) / 4) + (pl.wide ? 1 : 0);
   {

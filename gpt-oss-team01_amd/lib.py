@@ -102,6 +102,7 @@ SIGNATURES = {
     "gptoss_engine_destroy": (None, [_vp]),
     "gptoss_engine_tensor_view": (_i, [_vp, _i, _i, C.POINTER(_vp), C.POINTER(_sz)]),
     "gptoss_engine_debug_views": (_i, [_vp, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_sz)]),
+    "gptoss_diag_mfma_rate": (_i, [_i, _i, _i, _vp, C.POINTER(C.c_double), _vp]),
 }
 
 _lib = None

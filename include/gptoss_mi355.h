@@ -212,9 +212,14 @@ int gptoss_attn_decode_static(const float *q, const void *kv_cache, const int *l
 
 /* The same attention for T consecutive positions of every sequence at once (prompt processing):
  * q fp32 [B, T, n_q, D] and out bf16 [B, T, n_q, D]; row (b, t) attends to the cached positions up
- * to pos0 + t of sequence b, with the arithmetic gptoss_attn_decode uses for lens = pos0 + t + 1
- * and the same B, so its result is the one the T lock-step calls of the reference would give
- * (getp-csrc/submit/getp_run_submit.cpp:60-72 feeds prompts one position per step).  The cache must
+ * to pos0 + t of sequence b, with the arithmetic gptoss_attn_decode uses for lens = pos0 + t + 1,
+ * so its result is the one the T lock-step calls of the reference would give
+ * (getp-csrc/submit/getp_run_submit.cpp:60-72 feeds prompts one position per step): bit for bit
+ * for rows whose active positions span at most 512 cache slots; a longer row is summed block by
+ * block in one pass where the decode call merges partial sums, which can move the last bit of a
+ * few outputs.  With 32 or more positions per sequence (and at most 8 query heads per kv head) 16
+ * consecutive rows of a sequence share one pass over its K/V blocks, so a prompt of 1024 positions
+ * (the reference's cap, getp-csrc/src/alloc.cpp:1047) reads its cache 64 times, not 512.  The cache must
  * already hold positions [0, pos0 + T) of every sequence, all of them (a sliding-window ring
  * shorter than pos0 + T is refused: copy the prompt's K/V to a linear cache for this call). */
 size_t gptoss_attn_prefill_workspace_bytes(int B, int T, int n_q, int n_kv, int head_dim, int max_len);
@@ -378,6 +383,13 @@ enum {
   GPTOSS_TENSOR_B_ROUTER, GPTOSS_TENSOR_W1, GPTOSS_TENSOR_B1, GPTOSS_TENSOR_W2, GPTOSS_TENSOR_B2
 };
 int gptoss_engine_tensor_view(gptoss_engine *e, int tensor, int layer, void **ptr, size_t *bytes);
+
+/* Diagnostic without a counterpart in the reference: launches `workgroups` workgroups of 8 waves
+ * that each issue 4 * iters matrix instructions on operands held in registers (kind 0:
+ * v_mfma_f32_32x32x16_bf16; 1 / 2 / 3: v_mfma_scale_f32_32x32x64_f8f6f4 on fp8 x fp4, fp4 x fp4,
+ * fp8 x fp8 operands) and returns the flop the launch performs; the caller times it.  sink: 4
+ * bytes of device memory.  `python bench.py --mfma-rates` reports the rates. */
+int gptoss_diag_mfma_rate(int kind, int workgroups, int iters, float *sink, double *flop, void *stream);
 
 #ifdef __cplusplus
 }

@@ -199,11 +199,17 @@ def test_attn_batch_larger_than_one_launch_slice(ops, orc):
     (2, 65, 60, 64, 8, 64, 128),      # odd row count (the last row of a sequence has no partner), window edges
     (3, 41, 0, 8, 2, 32, 0),          # odd row count, four query heads per kv head
     (1, 66, 480, 64, 8, 64, 0),       # partners on either side of a chunk boundary (512 / 513 positions)
+    (1, 1024, 0, 64, 8, 64, 0),       # the reference's longest prompt: 16 blocks per row group
+    (2, 1024, 0, 8, 2, 32, 128),      # the same with the window, head_dim 32
+    (1, 1000, 24, 16, 2, 64, 128),    # row groups that start inside a block, 8 query heads per kv head, ragged end
+    (2, 20, 0, 8, 2, 32, 0),          # fewer than 32 positions: the row-pair form
 ])
 def test_attn_prefill_rows_equal_decode_calls(ops, orc, B, T, pos0, n_q, n_kv, D, window):
     """Prompt attention = the decode attention of every position at once: row (b, t) must equal, bit
     for bit, the decode call with lens = pos0 + t + 1 on the same cache (whatever else is in the
-    launch), and a sample of rows must match the oracle."""
+    launch) while the row's slot range fits one 512-slot chunk; a longer row is summed block by
+    block in one pass where the decode call merges chunk partials, so it may differ from it by a
+    last-bit rounding of a few outputs.  A sample of rows must match the oracle."""
     S = pos0 + T
     g = torch.Generator().manual_seed(S + n_q)
     q = torch.randn(B, T, n_q, D, generator=g)
@@ -224,7 +230,14 @@ def test_attn_prefill_rows_equal_decode_calls(ops, orc, B, T, pos0, n_q, n_kv, D
         lens = torch.full((B,), pos0 + t + 1, dtype=torch.int32)
         one = dec.forward(q[:, t].contiguous().cuda(), cache, lens.cuda(), sinks.cuda(), window=window,
                           max_len=pos0 + t + 1)
-        assert torch.equal(got[:, t], one), t
+        length = pos0 + t + 1
+        first_slot = (max(0, length - window) if window else 0) // 64 * 64
+        if length - first_slot <= 512:
+            assert torch.equal(got[:, t], one), t
+        else:
+            a, b = got[:, t].float(), one.float()
+            assert (a - b).abs().max() <= 2.0 ** -7 * b.abs().max(), t        # one bf16 step at the largest output
+            assert (a != b).float().mean() < 0.05, t
         want = orc.attn_decode(q[:, t].numpy(), K.float().numpy(), V.float().numpy(), lens.numpy(), sinks.numpy(),
                                window)
         mx, mean = rel_errors(got[:, t].float().cpu().numpy(), want)

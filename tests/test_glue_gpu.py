@@ -129,3 +129,26 @@ def test_rope_kv_store_then_attention(ops, orc, synth, D, n_q, n_kv):
     assert np.isfinite(got).all()
     mx, mean = rel_errors(got, want)
     assert mx <= TOL_MAX and mean <= TOL_MEAN, (mx, mean)
+
+
+def test_rope_kv_store_skips_empty_sequences(ops, orc, synth):
+    """lens[b] == 0 is an empty sequence, as for the attention call: its q row comes back zero and
+    nothing is written to its part of the cache; the other rows are unaffected."""
+    cfg = synth.tiny_config(2048)
+    D, n_q, n_kv, cap, B = cfg.head_dim, cfg.n_attn_heads, cfg.n_kv_heads, 64, 3
+    rng = np.random.default_rng(9)
+    qkv = torch.from_numpy(rng.standard_normal((B, (n_q + 2 * n_kv) * D)).astype(np.float32)).cuda()
+    cs, sn = orc.rope_tables(cfg, 8)
+    cs_d, sn_d = torch.from_numpy(cs).cuda(), torch.from_numpy(sn).cuda()
+    both = []
+    for lens in ([3, 0, 5], [3, 2, 5]):
+        cache = ops.KVCache(B, n_kv, D, cap)
+        cache.kv.view(torch.int16).fill_(0x1234)
+        q = ops.rope_kv_store(qkv, cache, cs_d, sn_d, torch.tensor(lens, dtype=torch.int32).cuda(), n_q)
+        torch.cuda.synchronize()
+        both.append((q.cpu().numpy(), cache.kv.view(torch.int16).cpu().numpy().reshape(B, -1)))
+    (q0, kv0), (q1, kv1) = both
+    assert (q0[1] == 0).all() and (kv0[1] == 0x1234).all()           # empty row: zero q, cache untouched
+    assert (kv1[1] != 0x1234).any()                                   # the same row with a length does store
+    for b in (0, 2):
+        assert np.array_equal(q0[b], q1[b]) and np.array_equal(kv0[b], kv1[b])
