@@ -34,6 +34,7 @@
 #include <type_traits>
 
 #include "common.hpp"
+#include "glue.hpp"
 
 namespace gptoss {
 
@@ -56,6 +57,7 @@ struct AttnParams {
   const int2 *order;   // workgroup-per-row kernel: (row, its length) by descending slot span (nullptr: row order)
   int2 *order_out;     // chunked kernels: when set, one extra workgroup (the last) writes that order
   int order_buckets;   // slot-span buckets (of 64 slots) the order distinguishes
+  const int *seq_map;  // optional: row b of a call with one row per sequence reads the cache of sequence seq_map[b]
 };
 
 // Cached positions of query row b: the caller's array, or the rule a host that knows every length
@@ -228,7 +230,8 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
   // behind the whole pass instead of sitting between the last block and the output store
   const float sink_logit = p.sinks ? p.sinks[head] : -INFINITY;
 
-  const int seq = (p.rows_per_seq > 1) ? b / p.rows_per_seq : b;
+  int seq = (p.rows_per_seq > 1) ? b / p.rows_per_seq : b;
+  if (p.seq_map) seq = __builtin_amdgcn_readfirstlane(p.seq_map[seq]);
   const bf16_t *plane = p.kv + kv_block_off(seq, g, p.n_kv, p.cap, D, 0);
   // lane's K bytes of a block: slot tb*16 + n, d chunk c*KS*8 .. +KS*8; its V bytes: 8 elements per
   // operand fragment
@@ -584,7 +587,9 @@ __global__ __launch_bounds__(TILE_WAVES * 64, 4) void attn_prefill_tile_kernel(A
   const int head = g * G + min(hn, G - 1);
   const float sink_logit = p.sinks ? p.sinks[head] : -INFINITY;
 
-  const unsigned char *plane = reinterpret_cast<const unsigned char *>(p.kv + kv_block_off(seq, g, p.n_kv, p.cap, D, 0));
+  const int cache_seq = p.seq_map ? __builtin_amdgcn_readfirstlane(p.seq_map[seq]) : seq;
+  const unsigned char *plane =
+      reinterpret_cast<const unsigned char *>(p.kv + kv_block_off(cache_seq, g, p.n_kv, p.cap, D, 0));
   // the workgroup's copy of a block: piece i of thread t is bytes (i * 512 + t) * 16; a K piece is
   // chunk j of row r and lands at chunk position j ^ swz(r) of its row, so that the 16 lanes of a
   // fragment read (16 rows, one chunk) hit 16 different 16-byte slots modulo 256 bytes
@@ -845,7 +850,8 @@ extern "C" size_t gptoss_attn_workspace_bytes(int B, int n_q, int n_kv, int head
 static int attn_launch(const float *q, const void *kv_cache, const int *lens,
                        const float *sinks, void *out, int B, int rows_per_seq, int n_q, int n_kv,
                        int head_dim, int capacity, int window, int max_len, void *workspace,
-                       size_t workspace_bytes, void *stream, int len_base = 0, int len_period = 0) {
+                       size_t workspace_bytes, void *stream, int len_base = 0, int len_period = 0,
+                       const int *seq_map = nullptr) {
   GPTOSS_REQUIRE(q && kv_cache && out, GPTOSS_ERR_NULL, "attn_decode: null pointer");
   if (!lens && len_base == 0) len_base = max_len;  // no lengths given: every row has max_len positions
   GPTOSS_REQUIRE(B > 0 && n_q > 0 && n_kv > 0 && n_q % n_kv == 0 && n_q / n_kv <= 16, GPTOSS_ERR_DIM,
@@ -891,6 +897,7 @@ static int attn_launch(const float *q, const void *kv_cache, const int *lens,
   p.order = nullptr;
   p.order_out = pl.wide ? order : nullptr;
   p.order_buckets = (span + 2 * ATT_BLOCK - 1) / ATT_BLOCK;
+  p.seq_map = seq_map;
   hipStream_t s = (hipStream_t)stream;
   // prompt passes put two consecutive rows of a sequence into one wave when the 16 operand columns
   // hold both rows' query heads and no ring can have wrapped (slot == position)
@@ -944,6 +951,13 @@ extern "C" int gptoss_attn_decode(const float *q, const void *kv_cache, const in
                                   int max_len, void *workspace, size_t workspace_bytes, void *stream) {
   return attn_launch(q, kv_cache, lens, sinks, out, B, 1, n_q, n_kv, head_dim, capacity, window,
                      max_len, workspace, workspace_bytes, stream);
+}
+
+int gptoss::attn_decode_mapped(const float *q, const void *kv_cache, const int *lens, const float *sinks, void *out,
+                               int B, int n_q, int n_kv, int head_dim, int capacity, int window, int max_len,
+                               void *workspace, size_t workspace_bytes, void *stream, const int *seq_map) {
+  return attn_launch(q, kv_cache, lens, sinks, out, B, 1, n_q, n_kv, head_dim, capacity, window, max_len, workspace,
+                     workspace_bytes, stream, 0, 0, seq_map);
 }
 
 // ---- the same call without a caller workspace ---------------------------------------------------
@@ -1004,6 +1018,7 @@ extern "C" size_t gptoss_attn_prefill_workspace_bytes(int B, int T, int n_q, int
 extern "C" int gptoss_attn_prefill(const float *q, const void *kv_cache, const float *sinks, void *out, int B, int T, int pos0, int n_q,
                                    int n_kv, int head_dim, int capacity, int window, void *workspace,
                                    size_t workspace_bytes, void *stream) {
+
   GPTOSS_REQUIRE(B > 0 && T > 0 && pos0 >= 0 && (long long)B * T < (1ll << 24), GPTOSS_ERR_DIM,
                  "attn_prefill: need B > 0, T > 0, pos0 >= 0 and B*T < 2^24 (B=%d T=%d)", B, T);
   GPTOSS_REQUIRE(window == 0 || pos0 + T <= capacity, GPTOSS_ERR_DIM,

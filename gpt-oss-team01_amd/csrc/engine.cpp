@@ -5,6 +5,7 @@
 // (getp-csrc/submit/getp_run_submit.cpp:13-96) or, by default, the same requests over a fixed set
 // of slots that are refilled as sequences end.
 #include <math.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include <algorithm>
@@ -70,7 +71,10 @@ struct gptoss_engine {
   // and a linear K/V scratch for the sliding-window layers when a prompt is longer than their ring
   struct Prefill {
     int rows;  // 0: not available
-    int *tokens;
+    int *tokens;          // [rows] followed by seq_map [rows], lens [rows], sample [max_batch]: one upload
+    int *seq_map, *lens;  // cache slot (and, for a step over arbitrary rows, cached positions) of every row
+    int *sample;          // rows whose next id is wanted
+    int *h_rows;          // pinned host image of tokens .. sample
     float *x, *qkv, *q, *tb2;
     bf16_t *t, *attn_out, *kv_scratch;
     size_t scratch_tokens;  // positions (summed over sequences) the scratch holds
@@ -329,6 +333,7 @@ void destroy(gptoss_engine *e) {
   for (void *p : e->allocs) (void)hipFree(p);
   if (e->h_tokens) (void)hipHostFree(e->h_tokens);
   if (e->h_next) (void)hipHostFree(e->h_next);
+  if (e->pf.h_rows) (void)hipHostFree(e->pf.h_rows);
   if (e->h_lens) (void)hipHostFree(e->h_lens);
   if (e->stream) (void)hipStreamDestroy(e->stream);
   delete e;
@@ -492,6 +497,7 @@ extern "C" int gptoss_engine_create(const gptoss_config *cfg, const float *host_
   e->h_tokens = e->h_next = e->h_lens = nullptr;
   e->stream = nullptr;
   e->pf.rows = 0;
+  e->pf.h_rows = nullptr;
   Builder b;
   b.e = e;
   b.hip(hipStreamCreate(&e->stream), "hipStreamCreate");
@@ -656,7 +662,12 @@ extern "C" int gptoss_engine_create(const gptoss_config *cfg, const float *host_
   if (!(flags & GPTOSS_ENGINE_NO_PREFILL)) {
     gptoss_engine::Prefill &pf = e->pf;
     const int R = (int)std::min<long long>((long long)max_batch * max_seq, PREFILL_ROWS);
-    pf.tokens = b.alloc<int>(R);
+    pf.tokens = b.alloc<int>((size_t)3 * R + max_batch);
+    pf.seq_map = pf.tokens + R;
+    pf.lens = pf.seq_map + R;
+    pf.sample = pf.lens + R;
+    b.hip(hipHostMalloc((void **)&pf.h_rows, sizeof(int) * ((size_t)3 * R + max_batch), hipHostMallocDefault),
+          "hipHostMalloc");
     pf.x = b.alloc<float>((size_t)R * H);
     pf.t = b.alloc<bf16_t>((size_t)R * H);
     pf.qkv = b.alloc<float>((size_t)R * qkv_dim);
@@ -894,6 +905,98 @@ extern "C" int gptoss_engine_prefill(gptoss_engine *e, const int *host_tokens, i
   return GPTOSS_OK;
 }
 
+// One step over n arbitrary rows: row i feeds token tok[i] at position pos[i] of the sequence in
+// cache slot slot[i].  Rows of one sequence must be consecutive positions in ascending order (a
+// stretch of its prompt): every row's K/V is stored before any row attends, and row i attends to
+// the positions up to its own.  On the sliding-window layers that is only correct while such a
+// stretch stays inside the ring's first lap (all its positions below the ring's capacity): the
+// caller sees to that.  The rows share every weight pass of the step, so the prompt of a request
+// that has just been admitted costs a few more rows in the GEMMs of a step that runs anyway.
+// host_next[j] = arg-max after row sample[j] (n_sample <= max_batch rows).
+static int step_rows(gptoss_engine *e, int n, const int *tok, const int *slot, const int *pos, int n_sample,
+                     const int *sample, int *host_next) {
+  const gptoss_config &c = e->cfg;
+  const int H = c.hidden_dim, V = c.vocab_size, L = c.n_layers, E = c.n_experts, k = c.experts_per_token;
+  const int D = c.head_dim, nq = c.n_attn_heads, nkv = c.n_kv_heads, I = c.intermediate_dim;
+  const int qkv_dim = (nq + 2 * nkv) * D;
+  gptoss_engine::Prefill &pf = e->pf;
+  GPTOSS_REQUIRE(n >= 1 && n <= pf.rows && n_sample >= 1 && n_sample <= e->max_batch, GPTOSS_ERR_DIM,
+                 "step_rows: %d rows (at most %d), %d sampled (at most %d)", n, pf.rows, n_sample, e->max_batch);
+  hipStream_t s = e->stream;
+  int rc;
+#define STEP(call)                   \
+  do {                               \
+    rc = (call);                     \
+    if (rc != GPTOSS_OK) return rc;  \
+  } while (0)
+  const size_t R = pf.rows;
+  int max_len = 1;
+  for (int i = 0; i < n; i++) {
+    pf.h_rows[i] = tok[i];
+    pf.h_rows[R + i] = slot[i];
+    pf.h_rows[2 * R + i] = pos[i] + 1;
+    max_len = std::max(max_len, pos[i] + 1);
+  }
+  for (int j = 0; j < n_sample; j++) pf.h_rows[3 * R + j] = sample[j];
+  // one copy when the rows are few enough that the gaps between the four arrays do not matter
+  if ((size_t)n * 8 >= R) {
+    GPTOSS_HIP(hipMemcpyAsync(pf.tokens, pf.h_rows, sizeof(int) * (3 * R + n_sample), hipMemcpyHostToDevice, s));
+  } else {
+    GPTOSS_HIP(hipMemcpyAsync(pf.tokens, pf.h_rows, sizeof(int) * n, hipMemcpyHostToDevice, s));
+    GPTOSS_HIP(hipMemcpyAsync(pf.seq_map, pf.h_rows + R, sizeof(int) * n, hipMemcpyHostToDevice, s));
+    GPTOSS_HIP(hipMemcpyAsync(pf.lens, pf.h_rows + 2 * R, sizeof(int) * n, hipMemcpyHostToDevice, s));
+    GPTOSS_HIP(hipMemcpyAsync(pf.sample, pf.h_rows + 3 * R, sizeof(int) * n_sample, hipMemcpyHostToDevice, s));
+  }
+  STEP(run_embedding(e->embedding, pf.tokens, pf.x, n, H, V, s));
+  for (int l = 0; l < L; l++) {
+    const LayerWeights &w = e->layers[l];
+    if (l == 0) STEP(run_rmsnorm(pf.x, nullptr, w.attn_norm, pf.t, nullptr, n, H, s));
+    STEP(dense_gemm(pf.t, w.w_qkv, w.b_qkv, pf.qkv, EPI_F32, n, qkv_dim, H, s));
+    STEP(run_rope_store_lens(pf.qkv, pf.q, w.kv_cache, e->cos_t, e->sin_t, n, nq, nkv, D, w.cache_cap, pf.lens, s,
+                             pf.seq_map));
+    STEP(attn_decode_mapped(pf.q, w.kv_cache, pf.lens, w.sinks, pf.attn_out, n, nq, nkv, D, w.cache_cap, w.window,
+                            max_len, pf.attn_ws, pf.attn_ws_bytes, s, pf.seq_map));
+    STEP(dense_gemm(pf.attn_out, w.w_o, w.b_o, pf.tb2, EPI_F32, n, H, nq * D, s));
+    STEP(run_rmsnorm(pf.x, pf.tb2, w.mlp_norm, pf.t, nullptr, n, H, s));
+    gptoss_moe_weights mw;
+    mw.n_experts = E;
+    mw.top_k = k;
+    mw.hidden = H;
+    mw.intermediate = I;
+    mw.swiglu_limit = c.swiglu_limit;
+    mw.w_router = w.w_router;
+    mw.b_router = w.b_router;
+    mw.w1 = w.w1;
+    mw.b1 = w.b1;
+    mw.w2 = w.w2;
+    mw.b2 = w.b2;
+    const float *nw = (l + 1 < L) ? e->layers[l + 1].attn_norm : nullptr;  // the sampled rows are normed below
+    const int q4 = (e->flags & GPTOSS_ENGINE_MXFP4_EXPERTS) ? 1 : 0;
+    const bool fused = nw && combine_norm_applies(H, nw, pf.t);
+    STEP(moe_forward_norm(&mw, pf.t, n, pf.x, pf.moe_ws, pf.moe_ws_bytes, s, q4, fused ? nw : nullptr,
+                          fused ? pf.t : nullptr));
+    if (nw && !fused) STEP(run_rmsnorm(pf.x, nullptr, nw, pf.t, nullptr, n, H, s));
+  }
+  STEP(run_gather_rows_idx(pf.x, e->x, pf.sample, n_sample, H, s));
+  STEP(run_rmsnorm(e->x, nullptr, e->final_norm, e->t, nullptr, n_sample, H, s));
+  if (e->logits) {
+    // the logits are kept per cache slot: one classifier row at a time
+    for (int j = 0; j < n_sample; j++) {
+      float *lg = e->logits + (size_t)slot[sample[j]] * V;
+      STEP(dense_gemm(e->t + (size_t)j * H, e->unembedding, nullptr, lg, EPI_F32, 1, V, H, s));
+      STEP(run_argmax(lg, e->d_next + j, 1, V, s));
+    }
+  } else {
+    STEP(dense_gemm(e->t, e->unembedding, nullptr, nullptr, EPI_ARGMAX, n_sample, V, H, s, e->amax_val, e->amax_idx));
+    STEP(run_argmax_tiles(e->amax_val, e->amax_idx, e->d_next, n_sample, gemm_col_tiles(V), s));
+  }
+  GPTOSS_HIP(hipMemcpyAsync(e->h_next, e->d_next, sizeof(int) * n_sample, hipMemcpyDeviceToHost, s));
+  GPTOSS_HIP(hipStreamSynchronize(s));
+  memcpy(host_next, e->h_next, sizeof(int) * n_sample);
+#undef STEP
+  return GPTOSS_OK;
+}
+
 // The reference's schedule: requests in batches of max_batch, every batch in lock step until its
 // last sequence ends (getp_run_submit.cpp:13-87).
 static int generate_lockstep(gptoss_engine *e, const int *host_prompts, const int *host_n_prompt,
@@ -965,10 +1068,19 @@ static int generate_lockstep(gptoss_engine *e, const int *host_prompts, const in
 }
 
 // Continuous batching: max_batch slots; a slot whose sequence ended (stop id or its length limit)
-// takes the next waiting request at once, at position 0, while the other slots carry on at their
-// own positions.  Every request sees the arithmetic it would see alone, so its output is the one
-// the lock-step schedule gives; only the order of the work changes.  host_max_len (optional) limits
-// request r to host_max_len[r] positions in all (prompt included) instead of max_seq_len.
+// takes the next waiting request at once, while the other slots carry on at their own positions.
+// Every request sees the arithmetic it would see alone, so its output is the one the lock-step
+// schedule gives; only the order of the work changes.  host_max_len (optional) limits request r
+// to host_max_len[r] positions in all (prompt included) instead of max_seq_len.
+//
+// Prompts are not forced one token per step (getp_run_submit.cpp:67-72 does that).  The positions
+// the first max_batch requests share go through one prompt pass; after that every step is a step
+// over rows (step_rows): one row for each sequence that is decoding, and for a request that has
+// just been admitted all the prompt positions it has left, as consecutive rows of the same step.
+// Those rows ride along in the weight passes the step makes anyway, so a prompt costs its slot
+// one step instead of one step per token.  On the sliding-window layers the rows of one step must
+// stay inside the first lap of the ring, so prompt positions from the ring's capacity on are
+// forced one per step as before; and a step never has more rows than the prompt buffers hold.
 static int generate_continuous(gptoss_engine *e, const int *host_prompts, const int *host_n_prompt,
                                int prompt_stride, int n_req, int max_seq_len, const int *host_max_len,
                                int *host_out, long long *n_generated) {
@@ -978,9 +1090,22 @@ static int generate_continuous(gptoss_engine *e, const int *host_prompts, const 
     if (n_generated) *n_generated = 0;
     return GPTOSS_OK;
   }
-  std::vector<int> req(B, -1), cur_tok(B, 0), cur_pos(B, 0), next(B);
+  std::vector<int> req(B, -1), cur_tok(B, 0), cur_pos(B, 0), next(B), prefix(B, 0);
   int next_req = 0, active_count = 0;
+  const bool rows_path = e->pf.rows > 0;
+  int ring_cap = e->max_seq + 1;  // positions a stretch of rows may reach on the window layers
+  for (const LayerWeights &w : e->layers)
+    if (w.window > 0) ring_cap = std::min(ring_cap, w.cache_cap);
   auto limit = [&](int r) { return host_max_len ? std::min(host_max_len[r], max_seq_len) : max_seq_len; };
+  // prompt positions of request r that may be run without looking at a result: a prompt's own stop
+  // token ends the sequence when it is fed, and the loop visits limit - 1 positions at most
+  auto forced_prefix = [&](int r) {
+    const int *pt = host_prompts + (size_t)r * prompt_stride;
+    int T = std::min(host_n_prompt[r], limit(r) - 1);
+    for (int j = 1; j < T; j++)
+      if (pt[j] == 199999 || pt[j] == 200002) T = j;
+    return T;
+  };
   auto finish = [&](int i) {
     const int r = req[i];
     int generated_len = cur_pos[i] - host_n_prompt[r];
@@ -998,57 +1123,96 @@ static int generate_continuous(gptoss_engine *e, const int *host_prompts, const 
       cur_tok[i] = host_prompts[(size_t)r * prompt_stride];
       cur_pos[i] = 0;
       active_count++;
-      if (limit(r) - 1 > 0) return;
+      if (limit(r) - 1 > 0) {
+        prefix[i] = forced_prefix(r);
+        return;
+      }
       finish(i);
     }
     cur_tok[i] = 0;
     cur_pos[i] = 0;
   };
+  // what the loop of getp_run_submit.cpp:60-96 does with the id the forward call of position
+  // cur_pos returned
+  auto advance = [&](int i, int next_id) {
+    const int r = req[i];
+    const int *pt = host_prompts + (size_t)r * prompt_stride;
+    const int np = host_n_prompt[r];
+    int *o = host_out + (size_t)r * (max_seq_len + 1);
+    int nt = next_id;
+    if (cur_pos[i] < np - 1) nt = pt[cur_pos[i] + 1];
+    else o[cur_pos[i] - (np - 1)] = nt;
+    cur_tok[i] = nt;
+    cur_pos[i]++;
+    if (nt == 199999 || nt == 200002 || cur_pos[i] >= limit(r) - 1) {
+      finish(i);
+      admit(i);
+    }
+  };
   for (int i = 0; i < B; i++) admit(i);
 
   // the prompt positions the first B requests share go through one prompt pass
-  bool first_wave = true;
+  bool first_wave = rows_path;
   for (int i = 0; i < B; i++) first_wave = first_wave && req[i] == i;
-  int skip_step = 0;
-  if (first_wave && e->pf.rows > 0) {
+  if (first_wave) {
     int T = e->pf.rows;
-    for (int i = 0; i < B; i++) {
-      const int *pt = host_prompts + (size_t)i * prompt_stride;
-      T = std::min(T, std::min(host_n_prompt[i], limit(i) - 1));
-      for (int j = 1; j < T; j++)
-        if (pt[j] == 199999 || pt[j] == 200002) T = j;
-    }
+    for (int i = 0; i < B; i++) T = std::min(T, prefix[i]);
     if (T >= 2) {
       std::vector<int> toks((size_t)B * T);
       for (int i = 0; i < B; i++)
         memcpy(&toks[(size_t)i * T], host_prompts + (size_t)i * prompt_stride, sizeof(int) * T);
       int rc = gptoss_engine_prefill(e, toks.data(), B, T, next.data());
       if (rc != GPTOSS_OK) return rc;
-      for (int i = 0; i < B; i++) cur_pos[i] = T - 1;  // the bookkeeping below finishes position T-1
-      skip_step = 1;
+      for (int i = 0; i < B; i++) cur_pos[i] = T - 1;  // advance() finishes position T-1
+      for (int i = 0; i < B; i++) advance(i, next[i]);
     }
   }
-  while (active_count > 0) {
-    if (!skip_step) {
+  if (!rows_path) {
+    while (active_count > 0) {
       int rc = gptoss_engine_step_ragged(e, cur_tok.data(), cur_pos.data(), B, next.data());
       if (rc != GPTOSS_OK) return rc;
+      for (int i = 0; i < B; i++)
+        if (req[i] >= 0) advance(i, next[i]);
     }
-    skip_step = 0;
+    if (n_generated) *n_generated = total;
+    return GPTOSS_OK;
+  }
+  std::vector<int> r_tok, r_slot, r_pos, sample, owner, count(B);
+  while (active_count > 0) {
+    // rows of this step: one per running sequence, plus what fits of the prompt stretches
+    int extra = e->pf.rows - active_count;
+    r_tok.clear();
+    r_slot.clear();
+    r_pos.clear();
+    sample.clear();
+    owner.clear();
     for (int i = 0; i < B; i++) {
-      const int r = req[i];
-      if (r < 0) continue;
-      const int *pt = host_prompts + (size_t)r * prompt_stride;
-      const int np = host_n_prompt[r];
-      int *o = host_out + (size_t)r * (max_seq_len + 1);
-      int nt = next[i];
-      if (cur_pos[i] < np - 1) nt = pt[cur_pos[i] + 1];
-      else o[cur_pos[i] - (np - 1)] = nt;
-      cur_tok[i] = nt;
-      cur_pos[i]++;
-      if (nt == 199999 || nt == 200002 || cur_pos[i] >= limit(r) - 1) {
-        finish(i);
-        admit(i);
+      count[i] = 0;
+      if (req[i] < 0) continue;
+      // positions cur_pos .. stretch_end - 1 are prompt positions whose inputs are known
+      const int stretch_end = std::min(prefix[i], ring_cap);
+      int m = 1;
+      if (cur_pos[i] + 1 < stretch_end) {
+        m = std::min(stretch_end - cur_pos[i], 1 + std::max(0, extra));
+        extra -= m - 1;
       }
+      const int *pt = host_prompts + (size_t)req[i] * prompt_stride;
+      for (int j = 0; j < m; j++) {
+        r_tok.push_back(j == 0 ? cur_tok[i] : pt[cur_pos[i] + j]);
+        r_slot.push_back(i);
+        r_pos.push_back(cur_pos[i] + j);
+      }
+      count[i] = m;
+      sample.push_back((int)r_tok.size() - 1);
+      owner.push_back(i);
+    }
+    int rc = step_rows(e, (int)r_tok.size(), r_tok.data(), r_slot.data(), r_pos.data(), (int)sample.size(),
+                       sample.data(), next.data());
+    if (rc != GPTOSS_OK) return rc;
+    for (size_t j = 0; j < owner.size(); j++) {
+      const int i = owner[j];
+      cur_pos[i] += count[i] - 1;  // advance() finishes the stretch's last position
+      advance(i, next[j]);
     }
   }
   if (n_generated) *n_generated = total;

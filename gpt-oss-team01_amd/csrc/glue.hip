@@ -112,12 +112,15 @@ __global__ __launch_bounds__(256) void rope_store_kernel(const float *__restrict
                                                          const float *__restrict__ cos_t,
                                                          const float *__restrict__ sin_t, int n_q,
                                                          int n_kv, int D, int cap, int pos0, int T,
-                                                         int store_from, const int *__restrict__ lens) {
+                                                         int store_from, const int *__restrict__ lens,
+                                                         const int *__restrict__ seq_map) {
   // row r of the batch is position pos0 + r % T of sequence r / T (T = 1: one lock-step position),
   // or, with lens, the last position (lens[r] - 1) of sequence r
+  // seq_map (optional): the cache of the r / T-th sequence of the batch is that of sequence seq_map[r / T]
   const int r = blockIdx.x;
-  const int b = r / T;
-  const int pos = lens ? lens[r] - 1 : pos0 + (r - b * T);
+  const int bi = r / T;
+  const int b = seq_map ? seq_map[bi] : bi;
+  const int pos = lens ? lens[r] - 1 : pos0 + (r - bi * T);
   if (pos < 0) {  // an empty sequence (lens[r] == 0): nothing to rotate or store, its q row is zero
     if (q_out != nullptr)
       for (int p = threadIdx.x; p < n_q * D; p += 256) q_out[(size_t)r * n_q * D + p] = 0.f;
@@ -332,7 +335,25 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(const float *__restric
     *reinterpret_cast<f32x4 *>(dp + i) = *reinterpret_cast<const f32x4 *>(sp + i);
 }
 
+// dst[i, :] = src[idx[i], :], n floats per row (n % 4 == 0)
+__global__ __launch_bounds__(256) void gather_rows_idx_kernel(const float *__restrict__ src,
+                                                              float *__restrict__ dst,
+                                                              const int *__restrict__ idx, int n) {
+  const float *sp = src + (size_t)idx[blockIdx.x] * n;
+  float *dp = dst + (size_t)blockIdx.x * n;
+  for (int i = threadIdx.x * 4; i < n; i += 256 * 4)
+    *reinterpret_cast<f32x4 *>(dp + i) = *reinterpret_cast<const f32x4 *>(sp + i);
+}
+
+int run_gather_rows_idx(const float *src, float *dst, const int *idx, int rows, int n, hipStream_t s) {
+  TraceScope ts("gather_rows", s);
+  gather_rows_idx_kernel<<<rows, 256, 0, s>>>(src, dst, idx, n);
+  GPTOSS_LAUNCH_CHECK("gather_rows_idx_kernel");
+  return GPTOSS_OK;
+}
+
 int run_gather_rows(const float *src, float *dst, int rows, int n, int stride, int offset, hipStream_t s) {
+  TraceScope ts("gather_rows", s);
   gather_rows_kernel<<<rows, 256, 0, s>>>(src, dst, n, stride, offset);
   GPTOSS_LAUNCH_CHECK("gather_rows_kernel");
   return GPTOSS_OK;
@@ -346,9 +367,9 @@ int run_rope_store(const float *qkv, float *q_out, bf16_t *kv, const float *cos_
 
 int run_rope_store_lens(const float *qkv, float *q_out, bf16_t *kv, const float *cos_t,
                         const float *sin_t, int B, int n_q, int n_kv, int D, int cap, const int *lens,
-                        hipStream_t s) {
+                        hipStream_t s, const int *seq_map) {
   TraceScope ts("rope_store", s);
-  rope_store_kernel<<<B, 256, 0, s>>>(qkv, q_out, kv, cos_t, sin_t, n_q, n_kv, D, cap, 0, 1, 0, lens);
+  rope_store_kernel<<<B, 256, 0, s>>>(qkv, q_out, kv, cos_t, sin_t, n_q, n_kv, D, cap, 0, 1, 0, lens, seq_map);
   GPTOSS_LAUNCH_CHECK("rope_store_kernel");
   return GPTOSS_OK;
 }
@@ -358,7 +379,7 @@ int run_rope_store_rows(const float *qkv, float *q_out, bf16_t *kv, const float 
                         int store_from, hipStream_t s) {
   TraceScope ts("rope_store", s);
   rope_store_kernel<<<rows, 256, 0, s>>>(qkv, q_out, kv, cos_t, sin_t, n_q, n_kv, D, cap, pos0, T,
-                                         store_from, nullptr);
+                                         store_from, nullptr, nullptr);
   GPTOSS_LAUNCH_CHECK("rope_store_kernel");
   return GPTOSS_OK;
 }

@@ -16,10 +16,18 @@ int run_rope_store(const float *qkv, float *q_out, bf16_t *kv, const float *cos_
 int run_rope_store_rows(const float *qkv, float *q_out, bf16_t *kv, const float *cos_t,
                         const float *sin_t, int rows, int T, int n_q, int n_kv, int D, int cap, int pos0,
                         int store_from, hipStream_t s);
-// one row per sequence, each at its own position lens[r] - 1
+// row r at position lens[r] - 1 of sequence r (or seq_map[r]: several rows may then belong to one
+// sequence, at different positions)
 int run_rope_store_lens(const float *qkv, float *q_out, bf16_t *kv, const float *cos_t,
                         const float *sin_t, int B, int n_q, int n_kv, int D, int cap, const int *lens,
-                        hipStream_t s);
+                        hipStream_t s, const int *seq_map = nullptr);
+// attn_decode.hip: gptoss_attn_decode with row b reading the cache of sequence seq_map[b] (device
+// array) up to lens[b]
+int attn_decode_mapped(const float *q, const void *kv_cache, const int *lens, const float *sinks, void *out, int B,
+                       int n_q, int n_kv, int head_dim, int capacity, int window, int max_len, void *workspace,
+                       size_t workspace_bytes, void *stream, const int *seq_map);
+// dst[i, :] = src[idx[i], :]
+int run_gather_rows_idx(const float *src, float *dst, const int *idx, int rows, int n, hipStream_t s);
 // dst[i, :] = src[i * stride + offset, :]
 int run_gather_rows(const float *src, float *dst, int rows, int n, int stride, int offset, hipStream_t s);
 int run_argmax(const float *logits, int *ids, int B, int V, hipStream_t s);

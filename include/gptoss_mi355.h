@@ -348,8 +348,13 @@ int gptoss_engine_prefill(gptoss_engine *e, const int *host_tokens, int B, int T
 /* Unless the engine was created with GPTOSS_ENGINE_PRECISE or GPTOSS_ENGINE_NO_PREFILL the
  * requests are scheduled continuously: max_batch slots, the prompt positions shared by the first
  * max_batch requests in one prompt pass, and a slot whose sequence ended (stop id or length limit)
- * takes the next waiting request at once.  Every request gets the arithmetic it would get alone, so
- * the output is that of the reference's batch-by-batch lock-step schedule. */
+ * takes the next waiting request at once.  A request admitted that way does not force its prompt
+ * one token per step (getp-csrc/submit/getp_run_submit.cpp:67-72): the prompt positions it has
+ * left run as consecutive rows of the next step, beside the one row of every sequence that is
+ * decoding, so they share that step's passes over the weights (on sliding-window layers only
+ * while they stay inside the ring's first lap; later prompt positions are forced as before).
+ * Every request gets the arithmetic it would get alone, so the output is that of the reference's
+ * batch-by-batch lock-step schedule. */
 int gptoss_engine_generate(gptoss_engine *e, const int *host_prompts, const int *host_n_prompt,
                            int prompt_stride, int n_req, int max_seq_len, int *host_out,
                            long long *n_generated);

@@ -386,6 +386,67 @@ def test_continuous_schedule_gives_the_lockstep_output(ops, tiny):
     assert n == total
 
 
+def test_continuous_schedule_runs_admitted_prompts_as_rows_of_a_step(ops, tiny):
+    """40 requests with prompts of 1..100 tokens and ragged limits over 6 slots.  A request admitted
+    into a slot that has become free runs all the prompt positions it has left as consecutive rows
+    of the next step, next to the single rows of the sequences that are decoding (every row's K/V
+    is stored before any row attends).  Outputs and token count must be exactly the lock-step
+    schedule's (rows are bit-equal to their lock-step steps: contexts below 512 positions, prompts
+    inside the first lap of the 128-slot ring), and the schedule must take far fewer steps than one
+    per position."""
+    fx, cfg, flat = tiny
+    rng = np.random.default_rng(17)
+    n_req, S = 40, 140
+    prompts = rng.integers(0, cfg.vocab_size, size=(n_req, 100)).astype(np.int32)
+    n_prompt = rng.integers(2, 101, size=n_req).astype(np.int32)
+    n_prompt[[4, 9]] = 1                                         # no stretch to run
+    max_len = np.minimum(S, n_prompt + rng.integers(1, 30, size=n_req)).astype(np.int32)
+    ref = ops.Engine(cfg, flat, max_batch=6, max_seq=S, prefill=False)
+    want, _ = ref.generate(prompts, S, n_prompt=n_prompt)
+    ref.close()
+    eng = ops.Engine(cfg, flat, max_batch=6, max_seq=S)
+    with ops.KernelTrace(capacity=16384) as tr:
+        got, n = eng.generate(prompts, S, n_prompt=n_prompt, max_len=max_len)
+    eng.close()
+    total = 0
+    for r in range(n_req):
+        gen = max(0, int(max_len[r]) - 1 - int(n_prompt[r]))
+        total += gen + 1
+        assert got[r, gen + 1] == -1, r
+        if gen > 0:
+            assert np.array_equal(got[r, :gen], want[r, :gen]), r
+    assert n == total
+    steps = sum(1 for name, _ in tr.results() if name == "embedding")   # one per step or pass
+    positions = int((max_len - 1).sum())
+    print("continuous schedule:", steps, "steps and passes for", positions, "positions on 6 slots")
+    assert steps < 0.5 * positions / 6, (steps, positions)
+
+
+def test_step_rows_stop_at_the_ring_capacity(ops, tiny, binfmt):
+    """Prompts longer than the sliding-window ring (here 64 slots holding a window of 8): a stretch
+    of rows may only cover the ring's first lap, the rest of the prompt is forced one position per
+    step.  The continuous schedule must still give the lock-step output."""
+    import dataclasses
+    fx, cfg0, flat = tiny
+    cfg = dataclasses.replace(cfg0, sliding_window=8)            # same tensors, a short window
+    rng = np.random.default_rng(23)
+    n_req, S = 10, 120
+    prompts = rng.integers(0, cfg.vocab_size, size=(n_req, 90)).astype(np.int32)
+    n_prompt = rng.integers(60, 91, size=n_req).astype(np.int32)
+    n_prompt[:3] = (40, 50, 45)        # the first three share a prompt pass: keep it inside the ring too
+    max_len = (n_prompt + rng.integers(2, 20, size=n_req)).astype(np.int32)
+    ref = ops.Engine(cfg, flat, max_batch=3, max_seq=S, prefill=False)
+    want, _ = ref.generate(prompts, S, n_prompt=n_prompt)
+    ref.close()
+    eng = ops.Engine(cfg, flat, max_batch=3, max_seq=S)
+    got, n = eng.generate(prompts, S, n_prompt=n_prompt, max_len=max_len)
+    eng.close()
+    for r in range(n_req):
+        gen = int(max_len[r]) - 1 - int(n_prompt[r])
+        assert got[r, gen + 1] == -1, r
+        assert np.array_equal(got[r, :gen], want[r, :gen]), r
+
+
 def test_stop_ids_in_prompts_and_schedules_agree(ops, orc, binfmt, synth):
     """A model with the real vocabulary size (so that the stop ids 199999 and 200002 exist) and
     prompts that contain them: a forced stop id ends its sequence in the reference's loop

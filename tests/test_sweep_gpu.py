@@ -84,9 +84,10 @@ def test_attn_random_shapes(ops, orc):
     print("random attention shapes: worst max-rel / mean-rel", worst)
 
 
-#: a router decision closer than this (k-th against (k+1)-th score, relative to the score scale of
-#: these models) may fall the other way under a different summation order
-ROUTER_NEAR_TIE = 3e-3
+#: a router decision of the staged CPU model closer than this (k-th against (k+1)-th score) may fall
+#: the other way on the GPU or under a different summation order: the criterion by which the
+#: lock-step comparison above drops rows.  (Observed flips: gaps of 3.1e-4 and 5.3e-3.)
+ROUTER_NEAR_TIE = 1.5e-2
 
 
 def _engine_case(ops, orc, binfmt, D, nq, nkv, H, E, k, I, L, V, win, B, T, seed, tok_cols):
