@@ -61,9 +61,12 @@ int run_router(const void *t, const void *w_router, const float *b_router, float
                int H, int E, int k, float *topk_w, int *topk_i, hipStream_t s);
 int run_topk_softmax(const float *logits, int B, int E, int k, float *topk_w, int *topk_i, hipStream_t s);
 // xcd_bounds (optional, XCD_BOUNDS_INTS + max_tiles ints): see GemmParams; tile_cost0_x2 = twice the fixed part of a tile's
-// cost in units of one 32-row block of arithmetic (cost = fixed + number of 32-row blocks)
+// cost in units of one 32-row block of arithmetic (cost = fixed + number of 32-row blocks);
+// sort_scratch (optional, group_sort_scratch_ints(B, k, E) ints): lets batches of 8192 pairs and more
+// be sorted by many workgroups
 int run_group(int B, int E, int k, float *topk_w, int *topk_i, int *expert_offsets,
               int *sorted_pair_ids, int *inv_perm, int *tiles, int rows_per_tile, int *xcd_bounds,
-              int tile_cost0_x2, hipStream_t s);
+              int tile_cost0_x2, hipStream_t s, int *sort_scratch = nullptr);
+inline size_t group_sort_scratch_ints(int B, int k, int E) { return (size_t)cdiv(B * k, 1024) * E; }
 
 }  // namespace gptoss

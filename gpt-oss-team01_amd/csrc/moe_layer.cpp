@@ -12,7 +12,7 @@ namespace gptoss {
 
 struct MoeWorkspace {
   float *logits, *topk_w;
-  int *topk_i, *expert_offsets, *sorted_pair_ids, *inv_perm, *tiles, *xcd_bounds;
+  int *topk_i, *expert_offsets, *sorted_pair_ids, *inv_perm, *tiles, *xcd_bounds, *sort_scratch;
   bf16_t *act;
   float *y2;
   size_t bytes;
@@ -35,6 +35,7 @@ static MoeWorkspace carve(void *base, int B, int E, int k, int H, int I) {
   w.inv_perm = (int *)take(P * 4);
   w.tiles = (int *)take((1 + 3 * (P / 32 + E)) * 4);
   w.xcd_bounds = (int *)take((XCD_BOUNDS_INTS + P / 32 + E) * 4);
+  w.sort_scratch = (int *)take(group_sort_scratch_ints(B, k, E) * 4);
   w.act = (bf16_t *)take(P * I * 2);
   w.y2 = (float *)take(P * H * 4);
   w.bytes = off;
@@ -142,7 +143,8 @@ static int moe_forward_impl(const gptoss_moe_weights *w, const void *t, int B, f
   rc = run_router(t, w->w_router, w->b_router, ws.logits, B, H, E, k, ws.topk_w, ws.topk_i, s);
   if (rc != GPTOSS_OK) return rc;
   rc = run_group(B, E, k, ws.topk_w, ws.topk_i, ws.expert_offsets, ws.sorted_pair_ids, ws.inv_perm,
-                 ws.tiles, rpt, ws.xcd_bounds, mxfp4 ? MOE_TILE_COST0_X2_MXFP4 : MOE_TILE_COST0_X2_BF16, s);
+                 ws.tiles, rpt, ws.xcd_bounds, mxfp4 ? MOE_TILE_COST0_X2_MXFP4 : MOE_TILE_COST0_X2_BF16, s,
+                 ws.sort_scratch);
   const int *bounds = max_tiles < 32768 ? ws.xcd_bounds : nullptr;
   if (rc != GPTOSS_OK) return rc;
 

@@ -209,6 +209,100 @@ __device__ __forceinline__ int wave_scan4(const int (&v)[4], int (&ex)[4]) {
   return __shfl(inc, 63, 64);
 }
 
+// From the experts' pair counts total[E] (LDS): the experts' offsets into offs[E+1] (LDS), and, when
+// `publish` is set, to memory together with the tile list, the tiles' blocks and the cut positions
+// of the work list.  Called by one whole wave (wave 0 of a workgroup); cost_pre / tile_pre are E
+// ints of LDS scratch each.
+__device__ __forceinline__ void group_finish(const int *total, int *offs, int *cost_pre, int *tile_pre, int E,
+                                             bool publish, int *__restrict__ expert_offsets,
+                                             int *__restrict__ tiles, int rows_per_tile,
+                                             int *__restrict__ xcd_bounds, int cost0) {
+  const int lane = threadIdx.x & 63;
+  int cnt[4], nt[4], off_ex[4], tile_ex[4];
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const int e = lane * 4 + i;
+    cnt[i] = (e < E) ? total[e] : 0;
+    nt[i] = (rows_per_tile > 0) ? (cnt[i] + rows_per_tile - 1) / rows_per_tile : 0;
+  }
+  const int all = wave_scan4(cnt, off_ex);
+  const int n_tiles = wave_scan4(nt, tile_ex);
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const int e = lane * 4 + i;
+    if (e < E) {
+      offs[e] = off_ex[i];
+      if (publish) expert_offsets[e] = off_ex[i];
+      if (publish && tiles != nullptr && rows_per_tile > 0) {
+        for (int t = 0; t < nt[i]; t++) {
+          int *tp = tiles + 1 + 3 * (tile_ex[i] + t);
+          tp[0] = e;
+          tp[1] = off_ex[i] + t * rows_per_tile;
+          tp[2] = min(rows_per_tile, cnt[i] - t * rows_per_tile);
+          // the block of up to MOE_TILE_BLOCK tiles of this expert that the tile belongs to
+          if (xcd_bounds != nullptr) {
+            const int b0 = t - t % MOE_TILE_BLOCK;
+            xcd_bounds[XCD_BOUNDS_INTS + tile_ex[i] + t] = ((tile_ex[i] + b0) << 8) | min(MOE_TILE_BLOCK, nt[i] - b0);
+          }
+        }
+      }
+    }
+  }
+  if (lane == 0) {
+    offs[E] = all;
+    if (publish) expert_offsets[E] = all;
+    if (publish && tiles != nullptr && rows_per_tile > 0) tiles[0] = n_tiles;
+  }
+  // Where to cut the tile list into 8 parts (one per XCD) of equal estimated cost: a tile costs
+  // cost0 + 2 per 32-row block (half units), all work items of a tile cost the same, and a cut may
+  // fall inside a tile (between two of its column tiles), hence the 16-bit fraction.
+  if (publish && xcd_bounds != nullptr && tiles != nullptr && rows_per_tile > 0) {
+    const int cfull = cost0 + 2 * (rows_per_tile / 32);
+    auto last_cost = [&](int count, int n) { return cost0 + 2 * ((count - (n - 1) * rows_per_tile + 31) / 32); };
+    int cost[4], cpre[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) cost[i] = (nt[i] > 0) ? (nt[i] - 1) * cfull + last_cost(cnt[i], nt[i]) : 0;
+    const int ctot = wave_scan4(cost, cpre);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const int e = lane * 4 + i;
+      if (e < E) {
+        cost_pre[e] = cpre[i];
+        tile_pre[e] = tile_ex[i];
+      }
+    }
+    // lane x finds cut x: the last expert whose cost prefix is <= x/8 of the total has a tile under
+    // the cut (experts without rows share their successor's prefix).  All quantities fit 32 bits:
+    // ctot < 2^15 tiles * (cost0 + 16).
+    if (lane < 8) {
+      int bound = 0;
+      if (ctot > 0) {
+        const int target = (lane * ctot) >> 3;
+        int lo = 0, hi = E - 1;
+        while (lo < hi) {
+          const int mid = (lo + hi + 1) >> 1;
+          if (cost_pre[mid] <= target) lo = mid;
+          else hi = mid - 1;
+        }
+        const int count = offs[lo + 1] - offs[lo];
+        const int nte = (count + rows_per_tile - 1) / rows_per_tile;
+        // float quotient (operands < 2^24) with a one-step correction instead of integer division
+        const int a = target - cost_pre[lo];
+        const float rcp_cfull = __builtin_amdgcn_rcpf((float)cfull);
+        int t = (int)((float)a * rcp_cfull);
+        t -= (t * cfull > a) ? 1 : 0;
+        t += ((t + 1) * cfull <= a) ? 1 : 0;
+        t = min(t, nte - 1);
+        const int rest = a - t * cfull;
+        const float inv = (t == nte - 1) ? __builtin_amdgcn_rcpf((float)last_cost(count, nte)) : rcp_cfull;
+        bound = ((tile_pre[lo] + t) << 16) | min(65535, (int)((float)rest * 65536.0f * inv));
+      }
+      xcd_bounds[lane] = bound;
+    }
+    if (lane == 0) xcd_bounds[8] = n_tiles << 16;
+  }
+}
+
 __global__ __launch_bounds__(SORT_THREADS) void group_sort_kernel(
     const int *__restrict__ topk_i, int P, int E, int nbits, int *__restrict__ expert_offsets,
     int *__restrict__ sorted_pair_ids, int *__restrict__ inv_perm, int *__restrict__ tiles,
@@ -267,92 +361,9 @@ __global__ __launch_bounds__(SORT_THREADS) void group_sort_kernel(
   }
   __syncthreads();
 
-  // expert offsets and first tile of every expert: two prefix sums over E <= 256 entries, wave 0
-  if (wave == 0) {
-    int cnt[4], nt[4], off_ex[4], tile_ex[4];
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-      const int e = lane * 4 + i;
-      cnt[i] = (e < E) ? total[e] : 0;
-      nt[i] = (rows_per_tile > 0) ? (cnt[i] + rows_per_tile - 1) / rows_per_tile : 0;
-    }
-    const int all = wave_scan4(cnt, off_ex);
-    const int n_tiles = wave_scan4(nt, tile_ex);
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-      const int e = lane * 4 + i;
-      if (e < E) {
-        offs[e] = off_ex[i];
-        expert_offsets[e] = off_ex[i];
-        if (tiles != nullptr && rows_per_tile > 0) {
-          for (int t = 0; t < nt[i]; t++) {
-            int *tp = tiles + 1 + 3 * (tile_ex[i] + t);
-            tp[0] = e;
-            tp[1] = off_ex[i] + t * rows_per_tile;
-            tp[2] = min(rows_per_tile, cnt[i] - t * rows_per_tile);
-            // the block of up to MOE_TILE_BLOCK tiles of this expert that the tile belongs to
-            if (xcd_bounds != nullptr) {
-              const int b0 = t - t % MOE_TILE_BLOCK;
-              xcd_bounds[XCD_BOUNDS_INTS + tile_ex[i] + t] = ((tile_ex[i] + b0) << 8) | min(MOE_TILE_BLOCK, nt[i] - b0);
-            }
-          }
-        }
-      }
-    }
-    if (lane == 0) {
-      offs[E] = all;
-      expert_offsets[E] = all;
-      if (tiles != nullptr && rows_per_tile > 0) tiles[0] = n_tiles;
-    }
-    // Where to cut the tile list into 8 parts (one per XCD) of equal estimated cost: a tile costs
-    // cost0 + 2 per 32-row block (half units), all work items of a tile cost the same, and a cut may
-    // fall inside a tile (between two of its column tiles), hence the 16-bit fraction.
-    if (xcd_bounds != nullptr && tiles != nullptr && rows_per_tile > 0) {
-      const int cfull = cost0 + 2 * (rows_per_tile / 32);
-      auto last_cost = [&](int count, int n) { return cost0 + 2 * ((count - (n - 1) * rows_per_tile + 31) / 32); };
-      int cost[4], cpre[4];
-#pragma unroll
-      for (int i = 0; i < 4; i++) cost[i] = (nt[i] > 0) ? (nt[i] - 1) * cfull + last_cost(cnt[i], nt[i]) : 0;
-      const int ctot = wave_scan4(cost, cpre);
-#pragma unroll
-      for (int i = 0; i < 4; i++) {
-        const int e = lane * 4 + i;
-        if (e < E) {
-          cost_pre[e] = cpre[i];
-          tile_pre[e] = tile_ex[i];
-        }
-      }
-      // lane x finds cut x: the last expert whose cost prefix is <= x/8 of the total has a tile under
-      // the cut (experts without rows share their successor's prefix).  All quantities fit 32 bits:
-      // ctot < 2^15 tiles * (cost0 + 16).
-      if (lane < 8) {
-        int bound = 0;
-        if (ctot > 0) {
-          const int target = (lane * ctot) >> 3;
-          int lo = 0, hi = E - 1;
-          while (lo < hi) {
-            const int mid = (lo + hi + 1) >> 1;
-            if (cost_pre[mid] <= target) lo = mid;
-            else hi = mid - 1;
-          }
-          const int count = offs[lo + 1] - offs[lo];
-          const int nte = (count + rows_per_tile - 1) / rows_per_tile;
-          // float quotient (operands < 2^24) with a one-step correction instead of integer division
-          const int a = target - cost_pre[lo];
-          const float rcp_cfull = __builtin_amdgcn_rcpf((float)cfull);
-          int t = (int)((float)a * rcp_cfull);
-          t -= (t * cfull > a) ? 1 : 0;
-          t += ((t + 1) * cfull <= a) ? 1 : 0;
-          t = min(t, nte - 1);
-          const int rest = a - t * cfull;
-          const float inv = (t == nte - 1) ? __builtin_amdgcn_rcpf((float)last_cost(count, nte)) : rcp_cfull;
-          bound = ((tile_pre[lo] + t) << 16) | min(65535, (int)((float)rest * 65536.0f * inv));
-        }
-        xcd_bounds[lane] = bound;
-      }
-      if (lane == 0) xcd_bounds[8] = n_tiles << 16;
-    }
-  }
+  // expert offsets, tile list and cut positions: wave 0
+  if (wave == 0)
+    group_finish(total, offs, cost_pre, tile_pre, E, true, expert_offsets, tiles, rows_per_tile, xcd_bounds, cost0);
   __syncthreads();
 
   for (int p0 = p_begin; p0 < p_end; p0 += 64 * SORT_CHUNK) {
@@ -374,6 +385,79 @@ __global__ __launch_bounds__(SORT_THREADS) void group_sort_kernel(
         if (valid && (mask & lt_mask) == 0) myhist[e[u]] += __popcll(mask);
       }
     }
+  }
+}
+
+
+// ---- the same sort by many workgroups (prompt passes, large batches) ---------------------------
+// One workgroup of 16 waves per 1024 pairs, one 64-pair step per wave.  First kernel: every pair's
+// rank among the pairs of its expert inside its workgroup (to rank[], which may be inv_perm) and
+// the workgroup's pair count per expert (wg_hist [G][E]).  Second kernel: every workgroup sums the
+// counts of the workgroups before it, derives the experts' offsets and scatters its pairs;
+// workgroup 0 also writes the offsets, the tile list and the cut positions.  The order inside an
+// expert is (workgroup, wave, lane) = pair order, as in the one-workgroup kernel.
+constexpr int SORT_PARALLEL_MIN_PAIRS = 8192;
+
+__global__ __launch_bounds__(SORT_THREADS) void group_count_kernel(const int *__restrict__ topk_i, int P, int E,
+                                                                   int nbits, int *__restrict__ wg_hist,
+                                                                   int *__restrict__ rank) {
+  extern __shared__ int smem[];  // [SORT_WAVES][E]
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const uint64_t lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+  for (int i = threadIdx.x; i < SORT_WAVES * E; i += SORT_THREADS) smem[i] = 0;
+  __syncthreads();
+  const int p = blockIdx.x * SORT_THREADS + threadIdx.x;
+  const int e = (p < P) ? topk_i[p] : -1;
+  const bool valid = (e >= 0 && e < E);
+  const uint64_t mask = same_expert_mask(e, valid, nbits);
+  if (valid && (mask & lt_mask) == 0) smem[wave * E + e] = __popcll(mask);
+  __syncthreads();
+  for (int x = threadIdx.x; x < E; x += SORT_THREADS) {
+    int run = 0;
+#pragma unroll
+    for (int w = 0; w < SORT_WAVES; w++) {
+      const int c = smem[w * E + x];
+      smem[w * E + x] = run;
+      run += c;
+    }
+    wg_hist[(size_t)blockIdx.x * E + x] = run;
+  }
+  __syncthreads();
+  if (valid) rank[p] = smem[wave * E + e] + __popcll(mask & lt_mask);
+}
+
+__global__ __launch_bounds__(SORT_THREADS) void group_scatter_kernel(
+    const int *__restrict__ topk_i, int P, int E, const int *__restrict__ wg_hist, const int *rank,
+    int *__restrict__ expert_offsets, int *__restrict__ sorted_pair_ids, int *inv_perm, int *__restrict__ tiles,
+    int rows_per_tile, int *__restrict__ xcd_bounds, int cost0) {
+  extern __shared__ int smem[];
+  int *before = smem;          // [E] pairs of the expert in the workgroups before this one
+  int *total = before + E;     // [E]
+  int *offs = total + E;       // [E+1]
+  int *cost_pre = offs + E + 1;
+  int *tile_pre = cost_pre + E;
+  const int wave = threadIdx.x >> 6;
+  const int G = gridDim.x;
+  for (int x = threadIdx.x; x < E; x += SORT_THREADS) {
+    int run = 0, mine = 0;
+    for (int g = 0; g < G; g++) {
+      if (g == (int)blockIdx.x) mine = run;
+      run += wg_hist[(size_t)g * E + x];
+    }
+    before[x] = mine;
+    total[x] = run;
+  }
+  __syncthreads();
+  if (wave == 0)
+    group_finish(total, offs, cost_pre, tile_pre, E, blockIdx.x == 0, expert_offsets, tiles, rows_per_tile,
+                 xcd_bounds, cost0);
+  __syncthreads();
+  const int p = blockIdx.x * SORT_THREADS + threadIdx.x;
+  const int e = (p < P) ? topk_i[p] : -1;
+  if (e >= 0 && e < E) {
+    const int dst = offs[e] + before[e] + rank[p];   // rank may alias inv_perm: read before the write below
+    sorted_pair_ids[dst] = p;
+    inv_perm[p] = dst;
   }
 }
 
@@ -436,28 +520,30 @@ extern "C" int gptoss_moe_max_tiles(int B, int k, int E, int rows_per_tile) {
 
 static int moe_route_impl(const float *logits, int B, int E, int k, float *topk_w, int *topk_i,
                           int *expert_offsets, int *sorted_pair_ids, int *inv_perm, int *tiles,
-                          int rows_per_tile, int *xcd_bounds, int tile_cost0_x2, void *stream, bool gate);
+                          int rows_per_tile, int *xcd_bounds, int tile_cost0_x2, void *stream, bool gate,
+                          int *sort_scratch);
 
 // grouping only: topk_i was already written by the fused router kernel
 int gptoss::run_group(int B, int E, int k, float *topk_w, int *topk_i, int *expert_offsets,
                       int *sorted_pair_ids, int *inv_perm, int *tiles, int rows_per_tile,
-                      int *xcd_bounds, int tile_cost0_x2, hipStream_t s) {
+                      int *xcd_bounds, int tile_cost0_x2, hipStream_t s, int *sort_scratch) {
   // the cut positions hold the tile index in 15 bits
   if (gptoss_moe_max_tiles(B, k, E, rows_per_tile) >= 32768) xcd_bounds = nullptr;
   return moe_route_impl(nullptr, B, E, k, topk_w, topk_i, expert_offsets, sorted_pair_ids, inv_perm,
-                        tiles, rows_per_tile, xcd_bounds, tile_cost0_x2, s, false);
+                        tiles, rows_per_tile, xcd_bounds, tile_cost0_x2, s, false, sort_scratch);
 }
 
 extern "C" int gptoss_moe_route(const float *logits, int B, int E, int k, float *topk_w,
                                 int *topk_i, int *expert_offsets, int *sorted_pair_ids,
                                 int *inv_perm, int *tiles, int rows_per_tile, void *stream) {
   return moe_route_impl(logits, B, E, k, topk_w, topk_i, expert_offsets, sorted_pair_ids, inv_perm,
-                        tiles, rows_per_tile, nullptr, 0, stream, true);
+                        tiles, rows_per_tile, nullptr, 0, stream, true, nullptr);
 }
 
 static int moe_route_impl(const float *logits, int B, int E, int k, float *topk_w, int *topk_i,
                           int *expert_offsets, int *sorted_pair_ids, int *inv_perm, int *tiles,
-                          int rows_per_tile, int *xcd_bounds, int tile_cost0_x2, void *stream, bool gate) {
+                          int rows_per_tile, int *xcd_bounds, int tile_cost0_x2, void *stream, bool gate,
+                          int *sort_scratch) {
   GPTOSS_REQUIRE(expert_offsets, GPTOSS_ERR_NULL, "moe_route: null pointer");
   GPTOSS_REQUIRE(B <= 0 || ((logits || !gate) && topk_w && topk_i && sorted_pair_ids && inv_perm),
                  GPTOSS_ERR_NULL, "moe_route: null pointer");
@@ -475,6 +561,19 @@ static int moe_route_impl(const float *logits, int B, int E, int k, float *topk_
   int nbits = 0;
   while ((1 << nbits) < E) nbits++;
   size_t smem = sizeof(int) * ((size_t)SORT_WAVES * E + E + (E + 1) + 2 * (size_t)E);
+  const int P = B * k;
+  if (sort_scratch != nullptr && P >= SORT_PARALLEL_MIN_PAIRS) {
+    const int G = cdiv(P, SORT_THREADS);
+    TraceScope ts("group_sort", s);
+    group_count_kernel<<<G, SORT_THREADS, sizeof(int) * SORT_WAVES * E, s>>>(topk_i, P, E, nbits, sort_scratch,
+                                                                           inv_perm);
+    GPTOSS_LAUNCH_CHECK("group_count_kernel");
+    group_scatter_kernel<<<G, SORT_THREADS, sizeof(int) * (5 * (size_t)E + 1), s>>>(
+        topk_i, P, E, sort_scratch, inv_perm, expert_offsets, sorted_pair_ids, inv_perm,
+        rows_per_tile ? tiles : nullptr, rows_per_tile, xcd_bounds, tile_cost0_x2);
+    GPTOSS_LAUNCH_CHECK("group_scatter_kernel");
+    return GPTOSS_OK;
+  }
   {
     TraceScope ts("group_sort", s);
     group_sort_kernel<<<1, SORT_THREADS, smem, s>>>(topk_i, B * k, E, nbits, expert_offsets,

@@ -248,3 +248,36 @@ def test_swiglu_special_cases_and_bias_order_through_a_one_expert_layer(ops, orc
     np.testing.assert_allclose(got[big_g], (sig7 * (uc_ + 1.0))[big_g], rtol=5e-3)
     np.testing.assert_allclose(got[big_g & (up < -7.0)], sig7 * -6.0, rtol=5e-3)
     assert (got[gate < -50] == 0).all()
+
+
+@pytest.mark.parametrize("B,E,k,skew", [(2048, 8, 4, 0.0), (2300, 40, 4, 2.0), (4096, 128, 4, 3.0), (3000, 256, 8, 0.0),
+                                        (9000, 32, 1, 1.0)])
+def test_grouping_by_many_workgroups(ops, orc, B, E, k, skew):
+    """From 8192 (token, expert) pairs on, the layer sorts them with one workgroup per 1024 pairs
+    (counts per workgroup, then offsets + scatter) instead of a single workgroup: offsets,
+    permutation and inverse must still be the stable counting sort, bit for bit, and the layer
+    output (which follows the tile list the same kernels write) must match the oracle."""
+    H = I = 64
+    g = torch.Generator().manual_seed(B + E)
+    n = lambda *s: _bf16(torch.randn(*s, generator=g) * 0.05)
+    br = _bf16(n(E).float() - skew * torch.arange(E) / E)
+    L = dict(w_router=n(E, H), b_router=br, w1=n(E, 2 * I, H), b1=n(E, 2 * I), w2=n(E, H, I), b2=n(E, H))
+    names = ("w_router", "b_router", "w1", "b1", "w2", "b2")
+    t = _bf16(torch.randn(B, H, generator=g))
+    layer = ops.MoeLayer(*[L[x].cuda() for x in names], top_k=k, max_tokens=B)
+    out = layer.forward(t.cuda())
+    torch.cuda.synchronize()
+    logits, tw, ti, off, srt, inv = [x.cpu().numpy() for x in layer.routing_views()]
+    assert B * k >= 8192
+    _, oi = orc.topk_softmax(logits, k)
+    ooff, osrt, oinv = orc.group(oi, E)
+    np.testing.assert_array_equal(ti, oi)
+    np.testing.assert_array_equal(off, ooff)
+    np.testing.assert_array_equal(srt, osrt)
+    np.testing.assert_array_equal(inv, oinv)
+    want, _, _, oti = orc.moe_layer(_f32np(t), *[_f32np(L[x]) for x in names], k=k, limit=7.0,
+                                    stage=orc.STAGE_SWIGLU, want_routing=True)
+    same = (oti == ti).all(axis=1)
+    assert same.mean() > 0.95
+    mx, mean = rel_errors(out.cpu().numpy()[same], want[same])
+    assert mx <= TOL_MAX and mean <= TOL_MEAN, (mx, mean)
