@@ -748,7 +748,7 @@ static int step_impl(gptoss_engine *e, const int *host_tokens, int pos, const in
                             w.cache_cap, w.window, pos + 1, e->attn_ws, e->attn_ws_bytes, s));
     STEP(dense_gemm(e->attn_out, w.w_o, w.b_o, e->tb2, EPI_F32, B, H, nq * D, s));
     // x += attention branch, then the ffn norm (model.cpp:66)
-    STEP(run_rmsnorm(e->x, e->tb2, w.mlp_norm, e->t, nullptr, B, H, s));
+    const MoePreNorm pre{e->x, e->tb2, w.mlp_norm};   // runs inside the block's router kernel
     gptoss_moe_weights mw;
     mw.n_experts = E;
     mw.top_k = k;
@@ -767,7 +767,7 @@ static int step_impl(gptoss_engine *e, const int *host_tokens, int pos, const in
     const int q4 = (e->flags & GPTOSS_ENGINE_MXFP4_EXPERTS) ? 1 : 0;
     const bool fused = combine_norm_applies(H, nw, e->t);
     STEP(moe_forward_norm(&mw, e->t, B, e->x, e->moe_ws, e->moe_ws_bytes, s, q4, fused ? nw : nullptr,
-                          fused ? e->t : nullptr));
+                          fused ? e->t : nullptr, &pre));
     if (!fused) STEP(run_rmsnorm(e->x, nullptr, nw, e->t, nullptr, B, H, s));
   }
   if (e->logits) {
@@ -850,7 +850,7 @@ static int prefill_chunk(gptoss_engine *e, const int *host_tokens, int seq0, int
                                pf.attn_ws, pf.attn_ws_bytes, s));
     }
     STEP(dense_gemm(pf.attn_out, w.w_o, w.b_o, pf.tb2, EPI_F32, rows, H, nq * D, s));
-    STEP(run_rmsnorm(pf.x, pf.tb2, w.mlp_norm, pf.t, nullptr, rows, H, s));
+    const MoePreNorm pre{pf.x, pf.tb2, w.mlp_norm};   // runs inside the block's router kernel
     gptoss_moe_weights mw;
     mw.n_experts = E;
     mw.top_k = k;
@@ -867,7 +867,7 @@ static int prefill_chunk(gptoss_engine *e, const int *host_tokens, int seq0, int
     const int q4 = (e->flags & GPTOSS_ENGINE_MXFP4_EXPERTS) ? 1 : 0;
     const bool fused = nw && combine_norm_applies(H, nw, pf.t);
     STEP(moe_forward_norm(&mw, pf.t, rows, pf.x, pf.moe_ws, pf.moe_ws_bytes, s, q4, fused ? nw : nullptr,
-                          fused ? pf.t : nullptr));
+                          fused ? pf.t : nullptr, &pre));
     if (nw && !fused) STEP(run_rmsnorm(pf.x, nullptr, nw, pf.t, nullptr, rows, H, s));
   }
   // only the last position of every sequence goes through the final norm and the classifier
@@ -957,7 +957,7 @@ static int step_rows(gptoss_engine *e, int n, const int *tok, const int *slot, c
     STEP(attn_decode_mapped(pf.q, w.kv_cache, pf.lens, w.sinks, pf.attn_out, n, nq, nkv, D, w.cache_cap, w.window,
                             max_len, pf.attn_ws, pf.attn_ws_bytes, s, pf.seq_map));
     STEP(dense_gemm(pf.attn_out, w.w_o, w.b_o, pf.tb2, EPI_F32, n, H, nq * D, s));
-    STEP(run_rmsnorm(pf.x, pf.tb2, w.mlp_norm, pf.t, nullptr, n, H, s));
+    const MoePreNorm pre{pf.x, pf.tb2, w.mlp_norm};   // runs inside the block's router kernel
     gptoss_moe_weights mw;
     mw.n_experts = E;
     mw.top_k = k;
@@ -974,7 +974,7 @@ static int step_rows(gptoss_engine *e, int n, const int *tok, const int *slot, c
     const int q4 = (e->flags & GPTOSS_ENGINE_MXFP4_EXPERTS) ? 1 : 0;
     const bool fused = nw && combine_norm_applies(H, nw, pf.t);
     STEP(moe_forward_norm(&mw, pf.t, n, pf.x, pf.moe_ws, pf.moe_ws_bytes, s, q4, fused ? nw : nullptr,
-                          fused ? pf.t : nullptr));
+                          fused ? pf.t : nullptr, &pre));
     if (nw && !fused) STEP(run_rmsnorm(pf.x, nullptr, nw, pf.t, nullptr, n, H, s));
   }
   STEP(run_gather_rows_idx(pf.x, e->x, pf.sample, n_sample, H, s));

@@ -47,10 +47,26 @@ int run_combine(const float *y2, const float *topk_w, const int *inv_perm, float
 inline bool combine_norm_applies(int H, const float *norm_w, const bf16_t *norm_out) {
   return norm_w && norm_out && H % 4 == 0 && H <= 4096 && aligned(norm_w, 16) && aligned(norm_out, 8);
 }
+// The norm in front of the MoE block, for the block to run itself: x += residual (residual may be
+// null), t = RMSNorm(x) * weight written to the block's input buffer.
+struct MoePreNorm {
+  float *x;
+  const float *residual;
+  const float *weight;
+};
 // The MoE block with the RMSNorm of the updated residual stream fused into its last kernel
-// (moe_layer.cpp); out is accumulated into.
+// (moe_layer.cpp); out is accumulated into.  With `pre`, t is an output of the call as well: the norm
+// that produces it runs inside the router kernel (or in a kernel of its own where that kernel's
+// limits do not allow it).
 int moe_forward_norm(const gptoss_moe_weights *w, const void *t, int B, float *out, void *workspace,
-                     size_t workspace_bytes, hipStream_t s, int mxfp4, const float *norm_w, bf16_t *norm_out);
+                     size_t workspace_bytes, hipStream_t s, int mxfp4, const float *norm_w, bf16_t *norm_out,
+                     const MoePreNorm *pre = nullptr);
+// moe_route.hip: residual add + RMSNorm + router GEMM + gating in one launch
+bool norm_router_applies(int B, int H, int E, const float *x, const float *residual, const float *weight,
+                         const void *t_out);
+int run_norm_router(float *x, const float *residual, const float *weight, void *t_out, const void *w_router,
+                    const float *b_router, float *logits, int B, int H, int E, int k, float *topk_w, int *topk_i,
+                    hipStream_t s);
 int moe_rows_per_tile(int B, int k, int E, bool mxfp4);
 // dense C = A . W^T (+ bias) with the epilogue `epi`; EPI_ARGMAX fills amax_val / amax_idx [B, gemm_col_tiles(N)]
 int dense_gemm(const bf16_t *A, const bf16_t *W, const float *bias, void *out, int epi, int B, int N, int K,

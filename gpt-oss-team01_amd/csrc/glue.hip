@@ -15,7 +15,19 @@ __global__ __launch_bounds__(256) void embedding_kernel(const bf16_t *__restrict
   int tok = tokens[b];
   tok = min(max(tok, 0), V - 1);
   const bf16_t *row = table + (size_t)tok * H;
-  for (int h = threadIdx.x; h < H; h += 256) x[(size_t)b * H + h] = bf16_to_f32(row[h]);
+  float *xr = x + (size_t)b * H;
+  if (H % 8 == 0 && reinterpret_cast<uintptr_t>(table) % 16 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0) {
+    // eight values per lane and step: one 16-byte load, two 16-byte stores
+    for (int h = threadIdx.x * 8; h < H; h += 256 * 8) {
+      const u32x4 v = *reinterpret_cast<const u32x4 *>(row + h);
+      *reinterpret_cast<f32x4 *>(xr + h) = f32x4{__uint_as_float(v[0] << 16), __uint_as_float(v[0] & 0xffff0000u),
+                                                 __uint_as_float(v[1] << 16), __uint_as_float(v[1] & 0xffff0000u)};
+      *reinterpret_cast<f32x4 *>(xr + h + 4) = f32x4{__uint_as_float(v[2] << 16), __uint_as_float(v[2] & 0xffff0000u),
+                                                     __uint_as_float(v[3] << 16), __uint_as_float(v[3] & 0xffff0000u)};
+    }
+    return;
+  }
+  for (int h = threadIdx.x; h < H; h += 256) xr[h] = bf16_to_f32(row[h]);
 }
 
 // RMSNorm with the arithmetic of run.cpp:304-317: sum of squares accumulated in double from

@@ -7,6 +7,7 @@
 
 #include "common.hpp"
 #include "gemm.hpp"
+#include "glue.hpp"
 
 namespace gptoss {
 
@@ -123,7 +124,8 @@ extern "C" int gptoss_moe_workspace_views(void *workspace, int B, int E, int k, 
 
 static int moe_forward_impl(const gptoss_moe_weights *w, const void *t, int B, float *out,
                             int accumulate, void *workspace, size_t workspace_bytes, void *stream,
-                            int mxfp4, const float *norm_w = nullptr, bf16_t *norm_out = nullptr) {
+                            int mxfp4, const float *norm_w = nullptr, bf16_t *norm_out = nullptr,
+                            const MoePreNorm *pre = nullptr) {
   int rc = check_moe(w, t, B, out, workspace, workspace_bytes);
   if (rc != GPTOSS_OK) return rc;
   if (B == 0) return GPTOSS_OK;
@@ -140,7 +142,17 @@ static int moe_forward_impl(const gptoss_moe_weights *w, const void *t, int B, f
   const int tile_block = MOE_TILE_BLOCK;
 
   // router GEMM with the gating of its own 16 tokens fused in, then the stable grouping
-  rc = run_router(t, w->w_router, w->b_router, ws.logits, B, H, E, k, ws.topk_w, ws.topk_i, s);
+  // (with `pre`, the residual add and RMSNorm that produce t run in the same launch)
+  if (pre && norm_router_applies(B, H, E, pre->x, pre->residual, pre->weight, t))
+    rc = run_norm_router(pre->x, pre->residual, pre->weight, const_cast<void *>(t), w->w_router, w->b_router,
+                         ws.logits, B, H, E, k, ws.topk_w, ws.topk_i, s);
+  else {
+    if (pre) {
+      rc = run_rmsnorm(pre->x, pre->residual, pre->weight, (bf16_t *)const_cast<void *>(t), nullptr, B, H, s);
+      if (rc != GPTOSS_OK) return rc;
+    }
+    rc = run_router(t, w->w_router, w->b_router, ws.logits, B, H, E, k, ws.topk_w, ws.topk_i, s);
+  }
   if (rc != GPTOSS_OK) return rc;
   rc = run_group(B, E, k, ws.topk_w, ws.topk_i, ws.expert_offsets, ws.sorted_pair_ids, ws.inv_perm,
                  ws.tiles, rpt, ws.xcd_bounds, mxfp4 ? MOE_TILE_COST0_X2_MXFP4 : MOE_TILE_COST0_X2_BF16, s,
@@ -186,8 +198,8 @@ static int moe_forward_impl(const gptoss_moe_weights *w, const void *t, int B, f
 
 int gptoss::moe_forward_norm(const gptoss_moe_weights *w, const void *t, int B, float *out, void *workspace,
                              size_t workspace_bytes, hipStream_t s, int mxfp4, const float *norm_w,
-                             bf16_t *norm_out) {
-  return moe_forward_impl(w, t, B, out, 1, workspace, workspace_bytes, s, mxfp4, norm_w, norm_out);
+                             bf16_t *norm_out, const MoePreNorm *pre) {
+  return moe_forward_impl(w, t, B, out, 1, workspace, workspace_bytes, s, mxfp4, norm_w, norm_out, pre);
 }
 
 extern "C" int gptoss_moe_forward(const gptoss_moe_weights *w, const void *t, int B, float *out,

@@ -2,6 +2,8 @@
 // shuffles, and a stable counting sort of the (token,slot) pairs by expert built from wave
 // ballots and an LDS histogram (no global atomics), which also emits the tile list that the
 // grouped GEMMs schedule from.
+#include <mutex>
+
 #include "common.hpp"
 #include "gemm.hpp"
 
@@ -80,18 +82,83 @@ constexpr int ROUTER_WAVES = 8;
 // so that a hidden size of 2880 with up to 32 experts is a single round of loads
 constexpr int router_steps(int nb) { return nb <= 2 ? 12 : (nb <= 4 ? 7 : (nb <= 8 ? 4 : 2)); }
 
-template <int NB>  // number of 16-expert column blocks held per wave
+// What the NORM form of the router kernel does first: x += residual, t = RMSNorm(x) * weight for the
+// workgroup's own token rows.
+struct RouterNorm {
+  float *x;               // [B,H] residual stream, updated in place
+  const float *residual;  // [B,H] or nullptr
+  const float *weight;    // [H]
+  bf16_t *t_out;          // [B,H]
+};
+
+// NB: number of 16-expert column blocks held per wave.  NORM: the workgroup first normalises its
+// rows (the arithmetic of rmsnorm_rows_kernel: 256 threads per row, the same element-to-thread
+// assignment and summation order, so t is the same to the bit), writes x and t to memory, keeps t in
+// LDS and multiplies from there: one launch and one read of t less than norm kernel + router kernel.
+template <int NB, bool NORM>
 __global__ __launch_bounds__(ROUTER_WAVES * 64) void router_gemm_kernel(
     const bf16_t *__restrict__ t, const bf16_t *__restrict__ wr, const float *__restrict__ br,
     float *__restrict__ logits, int B, int H, int E, int k, float *__restrict__ topk_w,
-    int *__restrict__ topk_i, int rows_per_wg) {
+    int *__restrict__ topk_i, int rows_per_wg, RouterNorm nrm) {
   __shared__ float red[ROUTER_WAVES][16][NB * 16 + 1];
+  extern __shared__ __attribute__((aligned(16))) unsigned char t_rows_raw[];  // NORM: [rows_per_wg][H] bf16
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   // rows_per_wg <= 16 token rows are this workgroup's; the other MFMA rows repeat the last of them
   const int r0 = blockIdx.x * rows_per_wg;
   const int arow = min(r0 + min(lane & 15, rows_per_wg - 1), B - 1);
   const int kq = (lane >> 4) * 8;
   const bf16_t *ap = t + (size_t)arow * H + kq;
+  if constexpr (NORM) {
+    constexpr int VPT = 4;  // rows of up to 4096 floats
+    __shared__ double nred[2][4];
+    bf16_t *t_rows = reinterpret_cast<bf16_t *>(t_rows_raw);
+    const int grp = threadIdx.x >> 8, tg = threadIdx.x & 255;  // two groups of 256 threads, a row each
+    for (int rr = 0; rr < rows_per_wg; rr += 2) {
+      const int lr = rr + grp;
+      const bool live = lr < rows_per_wg && r0 + lr < B;
+      const size_t row = (size_t)(r0 + lr) * H;
+      f32x4 v[VPT];
+      double ss = 0.0;
+#pragma unroll
+      for (int i = 0; i < VPT; i++) {
+        const int h = (tg + 256 * i) * 4;
+        v[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (live && h < H) {
+          v[i] = *reinterpret_cast<const f32x4 *>(nrm.x + row + h);
+          if (nrm.residual) {
+            const f32x4 r = *reinterpret_cast<const f32x4 *>(nrm.residual + row + h);
+#pragma unroll
+            for (int q = 0; q < 4; q++) v[i][q] = __fadd_rn(v[i][q], r[q]);
+            *reinterpret_cast<f32x4 *>(nrm.x + row + h) = v[i];
+          }
+#pragma unroll
+          for (int q = 0; q < 4; q++) ss += (double)__fmul_rn(v[i][q], v[i][q]);
+        }
+      }
+      for (int m = 32; m >= 1; m >>= 1) ss += __shfl_xor(ss, m, 64);
+      if (lane == 0) nred[grp][(threadIdx.x >> 6) & 3] = ss;
+      __syncthreads();
+      ss = nred[grp][0] + nred[grp][1] + nred[grp][2] + nred[grp][3];
+      ss /= H;
+      ss += 1e-5f;
+      const double inv = (double)(1.0f / sqrtf((float)ss));
+#pragma unroll
+      for (int i = 0; i < VPT; i++) {
+        const int h = (tg + 256 * i) * 4;
+        if (live && h < H) {
+          const f32x4 w = *reinterpret_cast<const f32x4 *>(nrm.weight + h);
+          f32x4 o;
+#pragma unroll
+          for (int q = 0; q < 4; q++) o[q] = (float)((double)w[q] * (inv * (double)v[i][q]));
+          const u32x2 pk = u32x2{pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3])};
+          *reinterpret_cast<u32x2 *>(nrm.t_out + row + h) = pk;
+          *reinterpret_cast<u32x2 *>(t_rows + (size_t)lr * H + h) = pk;
+        }
+      }
+      __syncthreads();   // nred is reused by the next pair of rows; after the last pair: t_rows complete
+    }
+    ap = t_rows + (size_t)(arow - r0) * H + kq;
+  }
   f32x4 acc[NB];
 #pragma unroll
   for (int nb = 0; nb < NB; nb++) acc[nb] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -475,6 +542,12 @@ int run_topk_softmax(const float *logits, int B, int E, int k, float *topk_w, in
   return GPTOSS_OK;
 }
 
+static int router_rows_per_wg(int B) {
+  int rows_per_wg = 16;
+  while (rows_per_wg > 4 && cdiv(B, rows_per_wg) < 256) rows_per_wg >>= 1;
+  return rows_per_wg;
+}
+
 // logits (+ optional gating of the same tokens) in one launch
 int run_router(const void *t, const void *w_router, const float *b_router, float *logits, int B,
                int H, int E, int k, float *topk_w, int *topk_i, hipStream_t s) {
@@ -482,19 +555,75 @@ int run_router(const void *t, const void *w_router, const float *b_router, float
   // with fewer rows each (the rest of the MFMA rows idle) all CUs take part in what is a
   // latency-bound launch: every workgroup reads the whole router matrix from L2 either way
   // (1024 tokens over 32 experts: 19.7 us with 16 rows, 16.7 with 8, 15.6 with 4, 27 with 2)
-  int rows_per_wg = 16;
-  while (rows_per_wg > 4 && cdiv(B, rows_per_wg) < 256) rows_per_wg >>= 1;
+  const int rows_per_wg = router_rows_per_wg(B);
   dim3 grid(cdiv(B, rows_per_wg)), block(ROUTER_WAVES * 64);
   const bf16_t *tp = (const bf16_t *)t, *wp = (const bf16_t *)w_router;
   int nb = cdiv(E, 16);
+  const RouterNorm none{nullptr, nullptr, nullptr, nullptr};
   TraceScope ts(topk_w ? "router_gemm_topk" : "router_gemm", s);
-  if (nb <= 1) router_gemm_kernel<1><<<grid, block, 0, s>>>(tp, wp, b_router, logits, B, H, E, k, topk_w, topk_i, rows_per_wg);
-  else if (nb <= 2) router_gemm_kernel<2><<<grid, block, 0, s>>>(tp, wp, b_router, logits, B, H, E, k, topk_w, topk_i, rows_per_wg);
-  else if (nb <= 4) router_gemm_kernel<4><<<grid, block, 0, s>>>(tp, wp, b_router, logits, B, H, E, k, topk_w, topk_i, rows_per_wg);
-  else if (nb <= 8) router_gemm_kernel<8><<<grid, block, 0, s>>>(tp, wp, b_router, logits, B, H, E, k, topk_w, topk_i, rows_per_wg);
-  else router_gemm_kernel<16><<<grid, block, 0, s>>>(tp, wp, b_router, logits, B, H, E, k, topk_w, topk_i, rows_per_wg);
+  if (nb <= 1) router_gemm_kernel<1, false><<<grid, block, 0, s>>>(tp, wp, b_router, logits, B, H, E, k, topk_w, topk_i, rows_per_wg, none);
+  else if (nb <= 2) router_gemm_kernel<2, false><<<grid, block, 0, s>>>(tp, wp, b_router, logits, B, H, E, k, topk_w, topk_i, rows_per_wg, none);
+  else if (nb <= 4) router_gemm_kernel<4, false><<<grid, block, 0, s>>>(tp, wp, b_router, logits, B, H, E, k, topk_w, topk_i, rows_per_wg, none);
+  else if (nb <= 8) router_gemm_kernel<8, false><<<grid, block, 0, s>>>(tp, wp, b_router, logits, B, H, E, k, topk_w, topk_i, rows_per_wg, none);
+  else router_gemm_kernel<16, false><<<grid, block, 0, s>>>(tp, wp, b_router, logits, B, H, E, k, topk_w, topk_i, rows_per_wg, none);
   GPTOSS_LAUNCH_CHECK("router_gemm_kernel");
   return GPTOSS_OK;
+}
+
+
+template <int NB>
+static int launch_norm_router(const RouterNorm &nrm, const bf16_t *wp, const float *b_router, float *logits, int B, int H,
+                              int E, int k, float *topk_w, int *topk_i, int rows_per_wg, size_t dyn, hipStream_t s) {
+  // the kernel's LDS (router partial sums + the rows of t) exceeds what a launch gets by default
+  constexpr int MAX_DEV = 64;
+  static std::mutex mu;
+  static size_t raised[MAX_DEV];
+  int dev = 0;
+  GPTOSS_HIP(hipGetDevice(&dev));
+  GPTOSS_REQUIRE(dev >= 0 && dev < MAX_DEV, GPTOSS_ERR_STATE, "router: device ordinal %d outside 0..%d", dev, MAX_DEV - 1);
+  auto kern = router_gemm_kernel<NB, true>;
+  {
+    std::lock_guard<std::mutex> lock(mu);
+    if (raised[dev] < dyn) {
+      GPTOSS_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                     (int)dyn));
+      raised[dev] = dyn;
+    }
+  }
+  TraceScope ts("norm_router_gemm_topk", s);
+  hipLaunchKernelGGL(kern, dim3(cdiv(B, rows_per_wg)), dim3(ROUTER_WAVES * 64), dyn, s, nrm.t_out, wp, b_router, logits, B,
+                     H, E, k, topk_w, topk_i, rows_per_wg, nrm);
+  GPTOSS_LAUNCH_CHECK("router_gemm_kernel (with norm)");
+  return GPTOSS_OK;
+}
+
+bool norm_router_applies(int B, int H, int E, const float *x, const float *residual, const float *weight,
+                         const void *t_out) {
+  const int nb = cdiv(E, 16) <= 1 ? 1 : cdiv(E, 16) <= 2 ? 2 : cdiv(E, 16) <= 4 ? 4 : cdiv(E, 16) <= 8 ? 8 : 16;
+  const size_t lds = (size_t)ROUTER_WAVES * 16 * (nb * 16 + 1) * 4 + (size_t)router_rows_per_wg(B) * H * 2 + 256;
+  // With more than four rows per workgroup (batches of more than ~1000 rows) the rows a workgroup
+  // normalises one after the other cost more than the launch the fusion saves (8192 rows: 2.58 ms
+  // per 24 layers against 2.23 ms for the two kernels; 1024 rows: 0.63 against 0.71 ms).
+  return B > 0 && router_rows_per_wg(B) <= 4 && H % 32 == 0 && H <= 4096 && lds <= 160 * 1024 && aligned(x, 16) && aligned(weight, 16) &&
+         aligned(t_out, 16) && (!residual || aligned(residual, 16));
+}
+
+// x += residual; t_out = RMSNorm(x) * weight; logits = t_out . Wr^T + br; gating: one launch
+int run_norm_router(float *x, const float *residual, const float *weight, void *t_out, const void *w_router,
+                    const float *b_router, float *logits, int B, int H, int E, int k, float *topk_w, int *topk_i,
+                    hipStream_t s) {
+  GPTOSS_REQUIRE(norm_router_applies(B, H, E, x, residual, weight, t_out), GPTOSS_ERR_DIM,
+                 "norm + router: shape or alignment outside the fused kernel's range (H=%d E=%d)", H, E);
+  const int rows_per_wg = router_rows_per_wg(B);
+  const RouterNorm nrm{x, residual, weight, (bf16_t *)t_out};
+  const bf16_t *wp = (const bf16_t *)w_router;
+  const size_t dyn = (size_t)rows_per_wg * H * 2;
+  const int nb = cdiv(E, 16);
+  if (nb <= 1) return launch_norm_router<1>(nrm, wp, b_router, logits, B, H, E, k, topk_w, topk_i, rows_per_wg, dyn, s);
+  if (nb <= 2) return launch_norm_router<2>(nrm, wp, b_router, logits, B, H, E, k, topk_w, topk_i, rows_per_wg, dyn, s);
+  if (nb <= 4) return launch_norm_router<4>(nrm, wp, b_router, logits, B, H, E, k, topk_w, topk_i, rows_per_wg, dyn, s);
+  if (nb <= 8) return launch_norm_router<8>(nrm, wp, b_router, logits, B, H, E, k, topk_w, topk_i, rows_per_wg, dyn, s);
+  return launch_norm_router<16>(nrm, wp, b_router, logits, B, H, E, k, topk_w, topk_i, rows_per_wg, dyn, s);
 }
 
 }  // namespace gptoss
