@@ -335,7 +335,8 @@ int gptoss_engine_step_ragged(gptoss_engine *e, const int *host_tokens, const in
 /* Positions 0..T-1 of B sequences in one pass: host_tokens int32 [B, T]; fills the KV caches and
  * returns in host_next[B] the arg-max ids after position T-1, i.e. what T calls of
  * gptoss_engine_step with pos = 0..T-1 leave behind (identical ids and caches while no
- * sliding-window ring has wrapped, equal to rounding after that).  Decoding continues with
+ * sliding-window ring has wrapped and the prompt has at most 512 positions; beyond either limit
+ * attention sums a row's scores in another order, so results are equal to rounding).  Decoding continues with
  * gptoss_engine_step at pos = T.  The reference has no such pass: it feeds prompts one position
  * per step (getp-csrc/submit/getp_run_submit.cpp:60-72).  Needs T <= max_seq and T <= 8192; not
  * available with GPTOSS_ENGINE_PRECISE or GPTOSS_ENGINE_NO_PREFILL. */
