@@ -997,6 +997,34 @@ static int step_rows(gptoss_engine *e, int n, const int *tok, const int *slot, c
   return GPTOSS_OK;
 }
 
+extern "C" int gptoss_engine_step_rows(gptoss_engine *e, int n_rows, const int *host_tokens, const int *host_slots,
+                                       const int *host_pos, int n_sample, const int *host_sample, int *host_next) {
+  GPTOSS_REQUIRE(e && host_tokens && host_slots && host_pos && host_sample && host_next, GPTOSS_ERR_NULL,
+                 "engine_step_rows: null pointer");
+  GPTOSS_REQUIRE(!(e->flags & GPTOSS_ENGINE_PRECISE) && e->pf.rows > 0, GPTOSS_ERR_STATE,
+                 "engine_step_rows: not available (GPTOSS_ENGINE_PRECISE or GPTOSS_ENGINE_NO_PREFILL)");
+  GPTOSS_REQUIRE(n_rows >= 1 && n_rows <= e->pf.rows && n_sample >= 1 && n_sample <= e->max_batch, GPTOSS_ERR_DIM,
+                 "engine_step_rows: %d rows outside 1..%d or %d sampled rows outside 1..%d", n_rows, e->pf.rows,
+                 n_sample, e->max_batch);
+  int ring_cap = e->max_seq + 1;
+  for (const LayerWeights &w : e->layers)
+    if (w.window > 0) ring_cap = std::min(ring_cap, w.cache_cap);
+  for (int i = 0; i < n_rows; i++) {
+    GPTOSS_REQUIRE(host_slots[i] >= 0 && host_slots[i] < e->max_batch && host_pos[i] >= 0 && host_pos[i] < e->max_seq,
+                   GPTOSS_ERR_STATE, "engine_step_rows: row %d names slot %d, position %d (slots 0..%d, positions 0..%d)",
+                   i, host_slots[i], host_pos[i], e->max_batch - 1, e->max_seq - 1);
+    // several rows of one sequence: consecutive, ascending, and inside the first lap of the window rings
+    if (i > 0 && host_slots[i] == host_slots[i - 1])
+      GPTOSS_REQUIRE(host_pos[i] == host_pos[i - 1] + 1 && host_pos[i] < ring_cap, GPTOSS_ERR_STATE,
+                     "engine_step_rows: rows %d and %d of slot %d must be consecutive positions below %d (got %d, %d)",
+                     i - 1, i, host_slots[i], ring_cap, host_pos[i - 1], host_pos[i]);
+  }
+  for (int j = 0; j < n_sample; j++)
+    GPTOSS_REQUIRE(host_sample[j] >= 0 && host_sample[j] < n_rows, GPTOSS_ERR_DIM,
+                   "engine_step_rows: sampled row %d outside 0..%d", host_sample[j], n_rows - 1);
+  return step_rows(e, n_rows, host_tokens, host_slots, host_pos, n_sample, host_sample, host_next);
+}
+
 // The reference's schedule: requests in batches of max_batch, every batch in lock step until its
 // last sequence ends (getp_run_submit.cpp:13-87).
 static int generate_lockstep(gptoss_engine *e, const int *host_prompts, const int *host_n_prompt,

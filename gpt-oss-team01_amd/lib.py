@@ -95,6 +95,7 @@ SIGNATURES = {
     "gptoss_engine_step": (_i, [_vp, _vp, _i, _i, _vp]),
     "gptoss_engine_prefill": (_i, [_vp, _vp, _i, _i, _vp]),
     "gptoss_engine_step_ragged": (_i, [_vp, _vp, _vp, _i, _vp]),
+    "gptoss_engine_step_rows": (_i, [_vp, _i, _vp, _vp, _vp, _i, _vp, _vp]),
     "gptoss_engine_generate_ragged": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp, _vp, C.POINTER(C.c_longlong)]),
     "gptoss_attn_prefill_workspace_bytes": (_sz, [_i, _i, _i, _i, _i, _i]),
     "gptoss_attn_prefill": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _sz, _vp]),

@@ -387,6 +387,18 @@ class Engine:
                                                   nxt.ctypes.data_as(C.c_void_p)))
         return nxt
 
+    def step_rows(self, tokens, slots, positions, sample):
+        """One step over arbitrary rows (token, cache slot, position); -> next ids after the rows `sample`."""
+        import numpy as np
+        tok = np.ascontiguousarray(tokens, dtype=np.int32)
+        slot = np.ascontiguousarray(slots, dtype=np.int32)
+        pos = np.ascontiguousarray(positions, dtype=np.int32)
+        smp = np.ascontiguousarray(sample, dtype=np.int32)
+        nxt = np.empty(smp.size, np.int32)
+        p = lambda a: a.ctypes.data_as(C.c_void_p)
+        _l.check(self.L.gptoss_engine_step_rows(self._h, tok.size, p(tok), p(slot), p(pos), smp.size, p(smp), p(nxt)))
+        return nxt
+
     def generate(self, prompts, max_seq_len, n_prompt=None, max_len=None):
         """Greedy generation; max_len (optional, per request) limits a request's total length."""
         import numpy as np

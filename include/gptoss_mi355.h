@@ -332,6 +332,21 @@ int gptoss_engine_step(gptoss_engine *e, const int *host_tokens, int pos, int B,
 int gptoss_engine_step_ragged(gptoss_engine *e, const int *host_tokens, const int *host_pos, int B,
                               int *host_next);
 
+/* One step over n_rows arbitrary rows: row i feeds host_tokens[i] at position host_pos[i] of the
+ * sequence in cache slot host_slots[i] (0 <= slot < max_batch).  Slots that have no row take no
+ * part in the step.  A slot may have several rows, a stretch of its prompt: they must be adjacent
+ * in the arrays, at consecutive ascending positions, and (with sliding-window layers) all below
+ * the window rings' capacity; every row's K/V is stored before any row attends and a row attends
+ * to the positions up to its own, so the stretch is processed as the same number of single steps
+ * would process it, inside one pass over the weights.  host_next[j] is the arg-max after row
+ * host_sample[j] (n_sample <= max_batch; the classifier runs for those rows only).  This is the
+ * step the continuous schedule of gptoss_engine_generate is made of; the reference has one
+ * position for the whole batch and one row per sequence
+ * (getp-csrc/src/model.cpp:6-151, submit/getp_run_submit.cpp:60-72).  n_rows <= 8192; not
+ * available with GPTOSS_ENGINE_PRECISE or GPTOSS_ENGINE_NO_PREFILL. */
+int gptoss_engine_step_rows(gptoss_engine *e, int n_rows, const int *host_tokens, const int *host_slots,
+                            const int *host_pos, int n_sample, const int *host_sample, int *host_next);
+
 /* Positions 0..T-1 of B sequences in one pass: host_tokens int32 [B, T]; fills the KV caches and
  * returns in host_next[B] the arg-max ids after position T-1, i.e. what T calls of
  * gptoss_engine_step with pos = 0..T-1 leave behind (identical ids and caches while no

@@ -114,6 +114,7 @@ def test_engine_entry_points_validate_before_touching_a_device(lib):
     # null engine / null buffers
     assert L.gptoss_engine_step(None, p, 0, 1, p) == 1
     assert L.gptoss_engine_step_ragged(None, p, p, 1, p) == 1
+    assert L.gptoss_engine_step_rows(None, 1, p, p, p, 1, p, p) == 1
     assert L.gptoss_engine_prefill(None, p, 1, 1, p) == 1
     n = C.c_longlong(0)
     assert L.gptoss_engine_generate(None, p, p, 1, 1, 8, p, C.byref(n)) == 1

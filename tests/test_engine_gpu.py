@@ -691,3 +691,42 @@ def test_prefill_of_1024_positions(ops, orc, tiny, synth, binfmt, head_dim, n_q,
     assert np.median(diffs) <= 5e-3, float(np.median(diffs))
     a.close()
     b.close()
+
+
+def test_step_rows_equals_single_steps(ops, tiny):
+    """gptoss_engine_step_rows directly: sequence 0 decodes at position 20, sequence 2 runs positions
+    0..11 of a prompt as twelve rows of the same step, slot 1 takes no part.  The sampled ids and the
+    logits must be those of the lock-step engine fed the same positions one by one, and bad row lists
+    are refused."""
+    from conftest import load_pkg
+    lib = load_pkg("lib")
+    fx, cfg, flat = tiny
+    rng = np.random.default_rng(31)
+    seq = rng.integers(0, cfg.vocab_size, size=(3, 40)).astype(np.int32)
+    a = ops.Engine(cfg, flat, max_batch=3, max_seq=64, keep_logits=True)
+    b = ops.Engine(cfg, flat, max_batch=3, max_seq=64, keep_logits=True)
+    for pos in range(20):                                    # sequence 0 up to position 19 in both engines
+        a.step(seq[:, pos], pos)
+        b.step(seq[:, pos], pos)
+    # lock-step reference: sequence 0 at position 20; sequence 2 restarted with a new prompt, 12 positions
+    prompt = rng.integers(0, cfg.vocab_size, size=12).astype(np.int32)
+    a.step_ragged(np.array([seq[0, 20], 0, prompt[0]], np.int32), np.array([20, 0, 0], np.int32))
+    want0 = a.last_logits(3)[0].copy()
+    for pos in range(1, 12):
+        a.step_ragged(np.array([seq[0, 20], 0, prompt[pos]], np.int32), np.array([20, 0, pos], np.int32))
+    want2 = a.last_logits(3)[2].copy()
+    tokens = np.concatenate([[seq[0, 20]], prompt]).astype(np.int32)
+    slots = np.array([0] + [2] * 12, np.int32)
+    poss = np.array([20] + list(range(12)), np.int32)
+    nxt = b.step_rows(tokens, slots, poss, sample=[0, 12])
+    lg = b.last_logits(3)
+    assert np.array_equal(lg[0], want0) and np.array_equal(lg[2], want2)
+    assert nxt.tolist() == [int(want0.argmax()), int(want2.argmax())]
+    with pytest.raises(lib.GptossError):                     # a stretch with a gap
+        b.step_rows(np.zeros(2, np.int32), np.array([1, 1], np.int32), np.array([0, 2], np.int32), sample=[1])
+    with pytest.raises(lib.GptossError):                     # slot outside the engine
+        b.step_rows(np.zeros(1, np.int32), np.array([3], np.int32), np.array([0], np.int32), sample=[0])
+    with pytest.raises(lib.GptossError):                     # sampled row outside the list
+        b.step_rows(np.zeros(1, np.int32), np.array([0], np.int32), np.array([0], np.int32), sample=[1])
+    a.close()
+    b.close()
