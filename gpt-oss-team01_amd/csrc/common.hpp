@@ -70,6 +70,17 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{lo, hi}, bf16x2));
 }
 
+// A pointer to data that nothing writes while the kernel runs, in the constant address space: a load
+// through it with a wave-uniform address is a scalar load whatever the kernel stores or clobbers
+// elsewhere (a generic pointer falls back to vector loads once the compiler sees a possible writer,
+// an asm statement with a memory clobber included).
+template <typename T>
+using const_as = const __attribute__((address_space(4))) T *;
+template <typename T>
+__device__ __forceinline__ const_as<T> constant_ptr(const T *q) {
+  return (const_as<T>)(q);
+}
+
 __device__ __forceinline__ bf16x8 as_bf16x8(u32x4 v) {
   union {
     u32x4 u;

@@ -35,10 +35,14 @@ struct GemmParams {
   float limit;         // SwiGLU clamp
 };
 
-// rows_per_tile in {32,64,96,128,160}; max_tiles bounds the number of
+// rows_per_tile in {32,64,96,128,160}, or 256 where gemm_tall_applies(); max_tiles bounds the number of
 // (mat,row-tile) items.
 int run_gemm(const GemmParams &p, bool gather, int epi, int rows_per_tile, int max_tiles,
              hipStream_t s);
+// gemm_tall.hip: tiles of 256 rows for launches of thousands of rows (bf16 weights; gather + SwiGLU or
+// plain fp32 output).  max_rows bounds the rows of A that the launch can address.
+bool gemm_tall_applies(const GemmParams &p, bool gather, int epi);
+int run_gemm_tall(const GemmParams &p, bool gather, int epi, int max_tiles, long long max_rows, hipStream_t s);
 // norm_w / norm_out (optional, accumulate only): also write RMSNorm(out) * norm_w as bf16.  Returns
 // with only the combine done when the fused form does not apply (H > 4096 or misaligned); the
 // caller checks with combine_norm_applies().

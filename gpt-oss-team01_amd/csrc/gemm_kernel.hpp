@@ -122,14 +122,17 @@ __device__ __forceinline__ void w_load(WRing<NRING, FP4> &ring, const WStream &s
 // store 8 or 16 bytes wide and keeps each (gate, up) pair inside a lane.
 // Biases are wave-uniform per register and half-wave: they come in through scalar loads, which
 // do not queue behind the vector loads already in flight for the next item.
-template <int MB, int EPI>
+// CONST_BIAS: read the biases through the constant address space, for a kernel whose asm statements
+// would otherwise turn these loads into vector loads.
+template <int MB, int EPI, bool CONST_BIAS = false>
 __device__ __forceinline__ void epilogue_store(const GemmParams &p, int mat, int row0, int rows, int n0,
                                                int lane, const f32x16 (&acc)[MB]) {
   const int N = p.N;
   const int tok = lane & 31;
   const bool hi = lane >= 32;
   const int h4 = hi ? 4 : 0;
-  const float *bp = p.bias ? p.bias + (size_t)mat * N + n0 : nullptr;
+  using BiasPtr = std::conditional_t<CONST_BIAS, const_as<float>, const float *>;
+  const BiasPtr bp = (BiasPtr)(p.bias ? p.bias + (size_t)mat * N + n0 : nullptr);
   if (EPI == EPI_SWIGLU) {
     // channels 0-15 of the wave are the gates of pairs j0..j0+15, channels 16-31 their ups; in the
     // unpacked matrix pair j is rows 2j (gate) and 2j+1 (up), so its biases are bp[2jj], bp[2jj+1]

@@ -1,5 +1,7 @@
 // Host side of the grouped/dense GEMMs (kernel dispatch), the weighted combine kernel and the
 // weight repacking kernels.  The GEMM kernel itself is in gemm_kernel.hpp.
+#include <stdlib.h>
+
 #include <mutex>
 
 #include "common.hpp"
@@ -252,6 +254,7 @@ int run_gemm(const GemmParams &p, bool gather, int epi, int rows_per_tile, int m
   const long long max_rows = p.tiles ? (long long)max_tiles * rows_per_tile : p.dense_rows;
   GPTOSS_REQUIRE(max_rows * p.N < (1ll << 32) && max_rows * p.K < (1ll << 32), GPTOSS_ERR_DIM,
                  "run_gemm: rows x columns must stay below 2^32 elements (rows<=%lld N=%d K=%d)", max_rows, p.N, p.K);
+  if (rows_per_tile == 256) return run_gemm_tall(p, gather, epi, max_tiles, max_rows, s);
   int prc = gemm_prepare_device();
   if (prc != GPTOSS_OK) return prc;
   if (gather && epi == EPI_SWIGLU) return dispatch_rows<true, EPI_SWIGLU>(p, rows_per_tile, max_tiles, s);
@@ -259,6 +262,16 @@ int run_gemm(const GemmParams &p, bool gather, int epi, int rows_per_tile, int m
   if (!gather && epi == EPI_ARGMAX && p.tiles == nullptr && p.amax_val && p.amax_idx)
     return dispatch_rows<false, EPI_ARGMAX>(p, rows_per_tile, max_tiles, s);
   return fail(GPTOSS_ERR_DIM, "run_gemm: unsupported combination (gather=%d epi=%d)", (int)gather, epi);
+}
+
+// rows from which a dense fp32-output GEMM uses the 256-row kernel of gemm_tall.hip
+static int dense_tall_min_rows() {
+  static const int v = [] {
+    const char *e = getenv("GPTOSS_DENSE_TALL_MIN_ROWS");
+    const int n = e ? atoi(e) : 0;
+    return n > 0 ? n : 2048;
+  }();
+  return v;
 }
 
 // C[B, N] = A[B, K] . W[N, K]^T (+ bias): the dense GEMMs of a step (QKV and output projections,
@@ -305,6 +318,7 @@ int dense_gemm(const bf16_t *A, const bf16_t *W, const float *bias, void *out, i
       }
     }
   }
+  if (B >= dense_tall_min_rows() && gemm_tall_applies(g, false, epi)) rpt = 256;
   return run_gemm(g, false, epi, rpt, cdiv(B, rpt), s);
 }
 

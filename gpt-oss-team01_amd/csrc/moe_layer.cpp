@@ -2,6 +2,7 @@
 // router GEMM -> top-k/softmax -> stable grouping + tile list -> grouped GEMM1 (+gather, +SwiGLU)
 // -> grouped GEMM2 -> ordered weighted combine.  Nothing here synchronises or allocates.
 #include <math.h>
+#include <stdlib.h>
 
 #include <algorithm>
 
@@ -52,6 +53,17 @@ static MoeWorkspace carve(void *base, int B, int E, int k, int H, int I) {
 // weights still come from HBM once.  96 rows only where they hold a whole expert; beyond that 64
 // (the 64-row kernel has room for a five-slab W ring, the 96-row one spills a few registers:
 // prompt passes of 8192 tokens 1.3 % faster with 64).
+static int env_int(const char *name, int dflt) {
+  const char *e = getenv(name);
+  const int n = e ? atoi(e) : 0;
+  return n > 0 ? n : dflt;
+}
+// average rows per expert from which a bf16 MoE block uses the 256-row kernels of gemm_tall.hip
+int moe_tall_min_rows() {
+  static const int v = env_int("GPTOSS_MOE_TALL_MIN_ROWS", 512);
+  return v;
+}
+
 int moe_rows_per_tile(int B, int k, int E, bool mxfp4) {
   double avg = (double)B * k / E;
   double need = avg + 2.5 * sqrt(avg);
@@ -132,7 +144,11 @@ static int moe_forward_impl(const gptoss_moe_weights *w, const void *t, int B, f
   const int E = w->n_experts, k = w->top_k, H = w->hidden, I = w->intermediate;
   hipStream_t s = (hipStream_t)stream;
   MoeWorkspace ws = carve(workspace, B, E, k, H, I);
-  const int rpt = moe_rows_per_tile(B, k, E, mxfp4 != 0);
+  int rpt = moe_rows_per_tile(B, k, E, mxfp4 != 0);
+  // a prompt pass, hundreds of rows per expert: bound by the matrix cores, not by streaming W
+  if (!mxfp4 && (long long)B * k >= (long long)moe_tall_min_rows() * E && H % 32 == 0 && H >= 256 && I % 32 == 0 &&
+      I >= 256)
+    rpt = 256;
   const int max_tiles = gptoss_moe_max_tiles(B, k, E, rpt);
   // Each expert's row tiles are walked in blocks of up to MOE_TILE_BLOCK, column tile by column
   // tile, so the workgroups of an XCD share a column tile of the expert's weights among the block's

@@ -44,8 +44,8 @@ def test_rmsnorm_matches_oracle(ops, orc, B, H):
                                         (600, 2880, 4096, True), (1024, 5120, 2880, False),
                                         (700, 4096, 256, True), (2304, 1056, 512, True)])
 def test_dense_gemm(ops, B, N, K, bias):
-    """Every regime of the dispatch: streaming kernel with 32..128-row tiles (B < 512) and the
-    compute-bound kernel with 128- and 256-row tiles, ragged last row tile and last column tile."""
+    """Every regime of the dispatch: row tiles of 32..160 rows chosen from the batch size, 256-row
+    tiles from 2048 rows on, ragged last row tile and last column tile."""
     g = torch.Generator(device="cuda").manual_seed(B + N)
     a = torch.randn(B, K, device="cuda", generator=g).to(torch.bfloat16)
     w = (torch.randn(N, K, device="cuda", generator=g) * 0.05).to(torch.bfloat16)
@@ -53,6 +53,21 @@ def test_dense_gemm(ops, B, N, K, bias):
     got = ops.dense_gemm(a, ops.pack_weight(w), N, b).cpu().numpy()
     want = (a.double() @ w.double().T + (b.double() if bias else 0)).cpu().numpy()
     assert np.abs(got - want).max() <= 2e-5 * np.abs(want).max() + 1e-6 * np.sqrt(K)
+
+
+@pytest.mark.parametrize("B,N,K", [(2500, 2880, 4096), (2049, 5120, 2880), (4096, 288, 256)])
+def test_dense_gemm_of_a_prompt_pass_equals_the_same_rows_in_small_batches(ops, B, N, K):
+    """From 2048 rows on the fp32 GEMM runs the kernel with 256-row tiles and both operands through
+    LDS: same bits per row as the streaming kernels, which run the batches of a fifth of the rows."""
+    g = torch.Generator(device="cuda").manual_seed(B + N)
+    a = torch.randn(B, K, device="cuda", generator=g).to(torch.bfloat16)
+    w = (torch.randn(N, K, device="cuda", generator=g) * 0.05).to(torch.bfloat16)
+    b = (torch.randn(N, device="cuda", generator=g)).to(torch.bfloat16).float()
+    wp = ops.pack_weight(w)
+    full = ops.dense_gemm(a, wp, N, b)
+    step = B // 5 + 1
+    for r0 in range(0, B, step):
+        assert torch.equal(full[r0:r0 + step], ops.dense_gemm(a[r0:r0 + step].contiguous(), wp, N, b)), r0
 
 
 @pytest.mark.parametrize("B,V,K", [(5, 4096, 256), (130, 201088, 2880), (1024, 50304, 512), (515, 9984, 256)])

@@ -281,3 +281,40 @@ def test_grouping_by_many_workgroups(ops, orc, B, E, k, skew):
     assert same.mean() > 0.95
     mx, mean = rel_errors(out.cpu().numpy()[same], want[same])
     assert mx <= TOL_MAX and mean <= TOL_MEAN, (mx, mean)
+
+
+# ---------------------------------------------------------------- prompt-pass sizes: 256-row tiles
+@pytest.mark.parametrize("B,E,H,I,skew", [
+    (2100, 8, 320, 320, 0.0),      # K = 320: ten stages; N = 640 and 320: a partial column tile each
+    (2600, 16, 256, 512, 1.1),     # skewed: experts of many tiles beside experts of a few rows
+    (1300, 4, 512, 256, 0.0),      # an expert's last tile of a few rows
+    (4100, 32, 2880, 2880, 0.0),   # the 20B layer at 4100 tokens
+])
+def test_moe_forward_of_a_prompt_pass_equals_the_same_tokens_in_small_batches(ops, orc, B, E, H, I, skew):
+    """From 512 rows per expert on average the block runs kernels of their own (256-row tiles, both
+    operands through LDS).  They must give every token the bits that the streaming kernels give it:
+    the full batch equals the same tokens run in batches of 1/8 of the size, and a sample equals the oracle."""
+    L = _rand_layer(E, H, I, 31)
+    if skew:
+        ranks = np.random.default_rng(B).permutation(E) + 1
+        L["b_router"] = torch.from_numpy((1.5 * np.log(1.0 / ranks ** skew)).astype(np.float32))
+    t = _bf16(torch.randn(B, H, generator=torch.Generator().manual_seed(B)))
+    layer = ops.MoeLayer(*[L[n].cuda() for n in ("w_router", "b_router", "w1", "b1", "w2", "b2")],
+                         max_tokens=B)
+    assert B * 4 >= 512 * E
+    full = layer.forward(t.cuda()).clone()
+    ti = layer.routing_views()[2].cpu().numpy()
+    step = B // 8 + 3
+    assert step * 4 < 512 * E
+    for r0 in range(0, B, step):
+        part = layer.forward(t[r0:r0 + step].cuda())
+        assert torch.equal(full[r0:r0 + step], part), r0
+    n_chk = 24
+    rows = np.r_[0:n_chk // 2, B - n_chk // 2:B]
+    want, _, _, oti = orc.moe_layer(_f32np(t)[rows], *[_f32np(L[n]) for n in
+                                    ("w_router", "b_router", "w1", "b1", "w2", "b2")],
+                                    k=4, limit=7.0, stage=orc.STAGE_SWIGLU, want_routing=True)
+    same = (oti == ti[rows]).all(axis=1)
+    assert same.mean() > 0.9
+    mx, mean = rel_errors(full.cpu().numpy()[rows][same], want[same])
+    assert mx <= TOL_MAX and mean <= TOL_MEAN, (mx, mean)
