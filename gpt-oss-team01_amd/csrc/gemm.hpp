@@ -39,8 +39,9 @@ struct GemmParams {
 // (mat,row-tile) items.
 int run_gemm(const GemmParams &p, bool gather, int epi, int rows_per_tile, int max_tiles,
              hipStream_t s);
-// gemm_tall.hip: tiles of 256 rows for launches of thousands of rows (bf16 weights; gather + SwiGLU or
-// plain fp32 output).  max_rows bounds the rows of A that the launch can address.
+// gemm_tall.hip: tiles of 256 x 256 with both operands through LDS, for launches of thousands of rows,
+// bound by the matrix cores (bf16 weights; gather + SwiGLU or plain fp32 output).  max_rows bounds
+// the rows of A that the launch can address.
 bool gemm_tall_applies(const GemmParams &p, bool gather, int epi);
 int run_gemm_tall(const GemmParams &p, bool gather, int epi, int max_tiles, long long max_rows, hipStream_t s);
 // norm_w / norm_out (optional, accumulate only): also write RMSNorm(out) * norm_w as bf16.  Returns

@@ -6,11 +6,15 @@
 // workgroup of four waves (one per SIMD) owns a 256 x 256 tile and a wave a 128 x 128 quarter of
 // it: 4 W fragments and 4 A fragments per k-step feed 16 MFMAs, half a fragment per MFMA.  Both
 // operands go from global memory straight into LDS with global_load_lds_dwordx4 (no staging
-// registers, no LDS store instructions) through four stages of 32 k; three stages are in flight;
-// the load pipeline runs on from one work item into the next.  W is read in the same packed
-// fragment order as everywhere else (a fragment lands in LDS as it is read); A rows are 64 bytes
-// per stage, their four 16-byte chunks XOR-swizzled by (row >> 1) & 3 so that fragment reads are
-// free of bank conflicts; the token gather of GEMM1 is a per-lane row offset of the load.
+// registers, no LDS store instructions), and the load pipeline runs on from one work item into
+// the next.
+//   W: stages of 32 k in four buffers, three in flight, in the same packed fragment order as
+//      everywhere else (a fragment lands in LDS as it is read).
+//   A: chunks of 64 k in three buffers, two in flight: a load instruction moves 8 rows x 128 bytes,
+//      whole cache lines.  (Rows of 64 bytes, one 32-k stage at a time, fetch every line twice, once per half:
+//      the loads of A then cost 2-3 times those of W, 55-65 us of a 265 us launch.)  The eight
+//      16-byte pieces of a row are XOR-swizzled by (row >> 1) & 7, so fragment reads are free of
+//      bank conflicts; the token gather of GEMM1 is a per-lane row offset of the load.
 // The loads are inline assembly, invisible to the compiler's wait counting, and the loop has no
 // other vector memory operation: every s_waitcnt vmcnt(N) is counted by hand (N = loads issued
 // behind the one waited for; stores of the previous item's epilogue that are still in flight only
@@ -24,30 +28,30 @@
 namespace gptoss {
 
 constexpr int TALL_THREADS = 256;
-constexpr int TALL_BM = 256, TALL_BN = 256, TALL_BK = 32;
-constexpr int TALL_STAGE = 32768;   // bytes: 8 column blocks x 2 k-steps x 1 KB of W, then 256 rows x 64 B of A
-constexpr int TALL_NST = 4;
-constexpr int TALL_IDS = TALL_NST * TALL_STAGE;  // behind the stages: 256 pair ids of the next item
-constexpr int TALL_LOADS = 8;       // load instructions per wave and stage: 2 x 2 of W, 4 of A
+constexpr int TALL_BK = 32;   // k of a W stage; an A chunk is two of them
+
+// A workgroup is WR x WC waves (four in all), a wave RB x CB blocks of 32 x 32 outputs.
+template <int WR_, int WC_, int RB_, int CB_>
+struct TallShape {
+  static_assert(WR_ * WC_ == 4, "four waves, one per SIMD");
+  static constexpr int WR = WR_, WC = WC_, RB = RB_, CB = CB_;
+  static constexpr int BM = WR * RB * 32, BN = WC * CB * 32;
+  static constexpr int NSTW = 4;                        // W stage buffers, NSTW - 1 in flight
+  static constexpr int W_BYTES = WC * CB * 2048;        // a W stage: a column block's two k-steps are 2 KB
+  static constexpr int A_BYTES = BM * 128;              // an A chunk: 128 bytes of every row
+  static constexpr int A_OFF = NSTW * W_BYTES;          // three A chunk buffers behind the W stages
+  static constexpr int SMEM = A_OFF + 3 * A_BYTES;      // 160 KB for the 256 x 256 tile: all of a CU's LDS
+  static constexpr int LW = WC * CB * 2 / 4;            // load instructions per wave: W fragments of a stage,
+  static constexpr int LA = BM / 8 / 4;                 // 8-row pieces of an A chunk
+  static_assert(WC * CB * 2 % 4 == 0 && BM % 32 == 0, "the loads are shared out evenly");
+  static_assert(SMEM <= 160 * 1024, "LDS of a CU");
+  static constexpr int NM = RB * CB, NR = RB + CB;      // MFMAs and fragment reads of a k-step
+  static_assert(LW % 2 == 0 && LA % 4 == 0, "a k-step issues half a W stage and a quarter of an A chunk");
+  static_assert(NM >= NR + 2 * (LA / 4 + LW / 2), "room for a k-step's reads and loads between its MFMAs");
+};
 
 __device__ __forceinline__ void tall_dma(unsigned lds_addr, uint32_t voff, const void *sbase) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(
-                   __builtin_amdgcn_readfirstlane(lds_addr)),
-               "v"(voff), "s"(sbase)
-               : "memory");
-}
-// two consecutive fragments (1 KB apart in memory and in LDS) with one M0
-__device__ __forceinline__ void tall_dma2(unsigned lds_addr, uint32_t voff, const void *sbase) {
-  asm volatile(
-      "s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2\n\tglobal_load_lds_dwordx4 %1, %2 offset:1024" ::"s"(
-          __builtin_amdgcn_readfirstlane(lds_addr)),
-      "v"(voff), "s"(sbase)
-      : "memory");
-}
-
-// the sorted pair ids of 64 rows of the NEXT work item, one per lane, into LDS through the same counted pipeline
-__device__ __forceinline__ void tall_dma_ids(unsigned lds_addr, uint32_t voff, const void *sbase) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(
                    __builtin_amdgcn_readfirstlane(lds_addr)),
                "v"(voff), "s"(sbase)
                : "memory");
@@ -64,28 +68,30 @@ __device__ __forceinline__ const T *uniform_ptr(const T *q) {
 }
 
 // where one work item's operands come from, for this wave's share of the loads
+template <class SH>
 struct TallSrc {
-  const unsigned char *w[2];  // first fragment of column blocks 2 wave, 2 wave + 1 of the tile
-  uint32_t a[4];              // byte offsets of this lane's chunk of its four A rows
+  const unsigned char *w[SH::LW];  // stage 0 of the W fragments this wave loads
+  uint32_t a[SH::LA];              // byte offsets of this lane's piece of the A rows it loads
   int mat, row0, rows, ct;
 };
 
-template <bool GATHER, int EPI>
+template <class SH, bool GATHER, int EPI>
 __global__ __launch_bounds__(TALL_THREADS, 1) void tall_gemm_kernel(GemmParams p) {
+  constexpr int RB = SH::RB, CB = SH::CB, LW = SH::LW, LA = SH::LA, LW1 = SH::LW / 2, LA1 = SH::LA / 4;
+  constexpr int NM = SH::NM, NR = SH::NR, NSTW = SH::NSTW;
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wr = w >> 1, wc = w & 1;   // the wave's 128 x 128 quarter of the tile
+  const int wr = w / SH::WC, wc = w % SH::WC;   // the wave's part of the tile
   const int K = p.K, N = p.N;
-  const int S = K / TALL_BK;
+  const int S = K / TALL_BK;                    // even: K % 64 == 0
   const unsigned lds_base =
       __builtin_amdgcn_readfirstlane((unsigned)(size_t)(__attribute__((address_space(3))) unsigned char *)lds);
   const unsigned char *abase = reinterpret_cast<const unsigned char *>(p.A);
-  const int *ids_lds = reinterpret_cast<const int *>(lds + TALL_IDS);
 
-  // ---- work list: the order of grouped_gemm_kernel (gemm_kernel.hpp), with 256-row tiles --------
+  // ---- work list: the order of grouped_gemm_kernel (gemm_kernel.hpp), with tiles of BM rows --------
   const const_as<int> tiles = constant_ptr(p.tiles), bounds = constant_ptr(p.xcd_bounds);
-  const int n_tiles = p.tiles ? tiles[0] : (p.dense_rows + TALL_BM - 1) / TALL_BM;
+  const int n_tiles = p.tiles ? tiles[0] : (p.dense_rows + SH::BM - 1) / SH::BM;
   const int total = n_tiles * p.n_col_tiles;
   const int per_xcd = gridDim.x >> 3;
   const int xcd = blockIdx.x & 7;
@@ -103,7 +109,7 @@ __global__ __launch_bounds__(TALL_THREADS, 1) void tall_gemm_kernel(GemmParams p
   auto valid = [&](int jj) { return lo + jj < hi; };
   if (!valid(j)) return;
   // which tile, which matrix, and this wave's share of the W loads
-  auto decode = [&](int jj, TallSrc &t) {
+  auto decode = [&](int jj, TallSrc<SH> &t) {
     const int work = lo + jj;
     int tile;
     if (p.tiles && p.tile_block > 1 && p.xcd_bounds) {
@@ -125,134 +131,183 @@ __global__ __launch_bounds__(TALL_THREADS, 1) void tall_gemm_kernel(GemmParams p
       t.rows = tiles[3 + 3 * tile];
     } else {
       t.mat = 0;
-      t.row0 = tile * TALL_BM;
-      t.rows = min(TALL_BM, p.dense_rows - t.row0);
+      t.row0 = tile * SH::BM;
+      t.rows = min(SH::BM, p.dense_rows - t.row0);
     }
     t.ct = __builtin_amdgcn_readfirstlane(t.ct);
     t.mat = __builtin_amdgcn_readfirstlane(t.mat);
     t.row0 = __builtin_amdgcn_readfirstlane(t.row0);
     t.rows = __builtin_amdgcn_readfirstlane(t.rows);
-    // this wave loads column blocks 2w and 2w+1 of the tile's eight (a block beyond N repeats the last one)
+    // W fragment f of a stage = (column block f / 2 of the tile, k-step f % 2); a block beyond N repeats the last one
     const unsigned char *wm = reinterpret_cast<const unsigned char *>(p.W) + (size_t)t.mat * N * K * 2;
 #pragma unroll
-    for (int q = 0; q < 2; q++) {
-      const int cb = min(t.ct * 8 + 2 * w + q, N / 32 - 1);
-      t.w[q] = uniform_ptr(wm + ((size_t)cb * (K / 16)) * 1024);
+    for (int q = 0; q < LW; q++) {
+      const int f = w * LW + q;
+      const int cb = min(t.ct * (SH::WC * CB) + (f >> 1), N / 32 - 1);
+      t.w[q] = uniform_ptr(wm + ((size_t)cb * (K / 16) + (f & 1)) * 1024);
     }
   };
-  // A: load instruction q of this wave moves tile rows (4w + q) * 16 .. + 16, four lanes per row and
-  // one 16-byte chunk per lane; rows past the tile's last one repeat it (their results are not stored)
-  auto a_offsets = [&](TallSrc &t, bool from_lds) {
+  // A: load instruction q of this wave moves 8 tile rows, eight lanes per row and one 16-byte piece
+  // per lane: the lane at position p of row r fetches piece p ^ ((r >> 1) & 7).  Rows past the
+  // tile's last one repeat it (their results are not stored).  The pair ids of a gathered tile are
+  // read through the constant address space: scalar loads, which the vector-memory counter of the
+  // hand-counted waits does not see.
+  auto a_offsets = [&](TallSrc<SH> &t) {
+    const const_as<int> ids = constant_ptr(p.row_ids);
 #pragma unroll
-    for (int q = 0; q < 4; q++) {
-      const int r = (w * 4 + q) * 16 + (lane >> 2);
+    for (int q = 0; q < LA; q++) {
+      const int r0 = (w * LA + q) * 8, r = r0 + (lane >> 3);
       int src;
-      if (GATHER) src = (from_lds ? ids_lds[r] : p.row_ids[t.row0 + min(r, t.rows - 1)]) / p.top_k;
-      else src = t.row0 + min(r, t.rows - 1);
-      const int c = (lane & 3) ^ ((r >> 1) & 3);
+      if (GATHER) {
+        src = ids[t.row0 + min(r0, t.rows - 1)];
+#pragma unroll
+        for (int i = 1; i < 8; i++) {
+          const int id = ids[t.row0 + min(r0 + i, t.rows - 1)];
+          src = (lane >> 3) == i ? id : src;
+        }
+        src /= p.top_k;
+      } else {
+        src = t.row0 + min(r, t.rows - 1);
+      }
+      const int c = (lane & 7) ^ ((r >> 1) & 7);
       t.a[q] = ((uint32_t)src * (uint32_t)K) * 2u + (uint32_t)c * 16u;
     }
   };
 
-  // one stage = 6 issue slots: 0, 1 = the two k-steps of W column block 2w + slot, 2..5 = A pieces
+  // W load instruction q of this wave for stage s of an item, into W buffer buf
   const uint32_t voff_w = lane * 16;
-  auto issue = [&](const TallSrc &t, int s, int buf, int slot) {
-    const unsigned sb = lds_base + buf * TALL_STAGE;
-    if (slot < 2) tall_dma2(sb + (2 * w + slot) * 2048, voff_w, t.w[slot] + (size_t)s * 2048);
-    else tall_dma(sb + 16384 + (w * 4 + slot - 2) * 1024, t.a[slot - 2], abase + (size_t)s * 64);
+  auto issue_w = [&](const TallSrc<SH> &t, int s, int buf, int q) {
+    tall_dma(lds_base + buf * SH::W_BYTES + (w * LW + q) * 1024, voff_w, t.w[q] + (size_t)s * 2048);
+  };
+  // A load instruction q of this wave for chunk c of an item, into A buffer buf
+  auto issue_a = [&](const TallSrc<SH> &t, int c, int buf, int q) {
+    tall_dma(lds_base + SH::A_OFF + buf * SH::A_BYTES + (w * LA + q) * 1024, t.a[q], abase + (size_t)c * 128);
   };
 
-  f32x16 acc[4][4];   // [column block][row block]
-  const int sw = ((lane & 31) >> 1) & 3, h = lane >> 5;
-  const unsigned a_rd = 16384 + (wr * 128 + (lane & 31)) * 64;
-  const unsigned a_k[2] = {(unsigned)(((0 + h) ^ sw) << 4), (unsigned)(((2 + h) ^ sw) << 4)};
-  const unsigned w_rd = (wc * 4) * 2 * 1024 + lane * 16;
-  bf16x8 F[2][8];     // two fragment sets: [0..3] W column blocks, [4..7] A row blocks
-  auto rd = [&](int buf, int kk, int set, int f) {
-    const unsigned char *sb = lds + buf * TALL_STAGE;
-    if (f < 4) F[set][f] = as_bf16x8(*reinterpret_cast<const u32x4 *>(sb + w_rd + (f * 2 + kk) * 1024));
-    else F[set][f] = as_bf16x8(*reinterpret_cast<const u32x4 *>(sb + a_rd + (f - 4) * 32 * 64 + a_k[kk]));
+  f32x16 acc[CB][RB];   // [column block][row block]
+  const int sw = ((lane & 31) >> 1) & 7, h = lane >> 5;
+  const unsigned a_rd = SH::A_OFF + (wr * RB * 32 + (lane & 31)) * 128;
+  unsigned a_k[4];      // where the lane finds its piece of k-step x of a chunk
+#pragma unroll
+  for (int x = 0; x < 4; x++) a_k[x] = (unsigned)(((2 * x + h) ^ sw) << 4);
+  const unsigned w_rd = (wc * CB) * 2 * 1024 + lane * 16;
+  bf16x8 F[2][NR];      // two fragment sets: [0, CB) W column blocks, [CB, CB + RB) A row blocks
+  // fragment read number i of a k-step, in the order the MFMAs want them: W0, every A, the other W;
+  // x = the k-step's number inside its A chunk
+  auto rd = [&](int wbuf, int kk, int abuf, int x, int set, int i) {
+    const int f = i == 0 ? 0 : (i <= RB ? CB + i - 1 : i - RB);
+    if (f < CB)
+      F[set][f] = as_bf16x8(*reinterpret_cast<const u32x4 *>(lds + wbuf * SH::W_BYTES + w_rd + (f * 2 + kk) * 1024));
+    else
+      F[set][f] = as_bf16x8(
+          *reinterpret_cast<const u32x4 *>(lds + abuf * SH::A_BYTES + a_rd + (f - CB) * 32 * 128 + a_k[x]));
   };
-  constexpr int RO[8] = {0, 4, 5, 6, 7, 1, 2, 3};  // read order: what the first MFMAs need first
+  // one k-step: NM MFMAs out of fragment set `set`; with the first NR of them the fragment reads of
+  // the next k-step (into the other set), behind those whatever loads `loads(m)` issues
+  auto kstep = [&](int set, int wbuf, int kk, int abuf, int x, auto &&loads) {
+#pragma unroll
+    for (int m = 0; m < NM; m++) {
+      acc[m / RB][m % RB] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(F[set][m / RB], F[set][CB + m % RB],
+                                                                    acc[m / RB][m % RB], 0, 0, 0);
+      if (m < NR) rd(wbuf, kk, abuf, x, set ^ 1, m);
+      loads(m);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
 
-  TallSrc cur, nxt;
+  TallSrc<SH> cur, nxt;
   decode(j, cur);
-  a_offsets(cur, false);
+  a_offsets(cur);
+  // The first loads go out in the order the stage loop would have issued them, so that its waits
+  // count right from the first stage on: chunk 0 and W stage 0, then a quarter of chunk 1 with
+  // every half of W stages 1 and 2.
 #pragma unroll
-  for (int q = 0; q < 3; q++)
+  for (int q = 0; q < LA; q++) issue_a(cur, 0, 0, q);
 #pragma unroll
-    for (int m = 0; m < 6; m++) issue(cur, q, q, m);
-  wait_vmcnt<2 * TALL_LOADS>();   // stage 0 has landed; stages 1 and 2 may be on their way
+  for (int q = 0; q < LW; q++) issue_w(cur, 0, 0, q);
+#pragma unroll
+  for (int x = 0; x < 4; x++) {
+#pragma unroll
+    for (int q = 0; q < LA1; q++) issue_a(cur, 1, 1, x * LA1 + q);
+#pragma unroll
+    for (int q = 0; q < LW1; q++) issue_w(cur, 1 + (x >> 1), 1 + (x >> 1), (x & 1) * LW1 + q);
+  }
+  wait_vmcnt<4 * (LA1 + LW1)>();   // chunk 0 and stage 0 have landed; the loads behind them may be on their way
   __builtin_amdgcn_s_barrier();
 #pragma unroll
-  for (int f = 0; f < 8; f++) rd(0, 0, 0, RO[f]);
+  for (int i = 0; i < NR; i++) rd(0, 0, 0, 0, 0, i);
   __builtin_amdgcn_sched_barrier(0);
-  int g = 0;  // running stage count: the buffer of a stage is its count & 3
+  int g = 0;   // running stage count (even at the start of every item): W buffer g & 3
+  int ab = 0;  // A buffer of the current chunk: the running chunk count modulo 3
   while (true) {
     const int jn = j + per_xcd;
     const bool more = valid(jn);
-    nxt = cur;  // past the last item the pipeline requests this item's first stages again, and drops them
+    nxt = cur;  // past the last item the pipeline requests this item's first loads again, and drops them
     if (more) {
       decode(jn, nxt);
-      if (GATHER) {
-        // One more load in the queue, in front of the five of stage g+3: the wait of this stage is one
-        // load stricter than it needs to be, and the wait of the next stage (13 younger loads) covers
-        // this load, so the ids are in LDS, written and read by this wave alone, from stage 2 on.
-        const int r = min(w * 64 + lane, nxt.rows - 1);
-        tall_dma_ids(lds_base + TALL_IDS + w * 256, (uint32_t)r * 4u, uniform_ptr(p.row_ids + nxt.row0));
-      } else {
-        a_offsets(nxt, false);
-      }
+      a_offsets(nxt);
     }
 #pragma unroll
-    for (int i = 0; i < 4; i++)
+    for (int i = 0; i < CB; i++)
 #pragma unroll
-      for (int r = 0; r < 4; r++)
+      for (int r = 0; r < RB; r++)
 #pragma unroll
         for (int x = 0; x < 16; x++) acc[i][r][x] = 0.f;
-    for (int s = 0; s < S; s++, g++) {
-      if (GATHER && s == 2 && more) a_offsets(nxt, true);
-      const int cb = g & 3, nb = (g + 1) & 3, pb = (g + 3) & 3;
-      const bool wrap = s + 3 >= S;
-      const int s3 = wrap ? s + 3 - S : s + 3;
-      TallSrc src;
+    for (int s = 0; s < S; s += 2, g += 2) {
+      // ---- even stage s: the first half of A chunk s / 2 --------------------------------------
+      const int ab1 = ab == 2 ? 0 : ab + 1, ab2 = ab1 == 2 ? 0 : ab1 + 1;
+      const bool wrap_a = s + 4 >= S;             // the chunk requested now: two ahead, or one of the next item's first two
+      const bool wrap_w0 = s + 3 >= S, wrap_w1 = s + 4 >= S;
+      TallSrc<SH> sa, s0, s1;
 #pragma unroll
-      for (int q = 0; q < 2; q++) src.w[q] = wrap ? nxt.w[q] : cur.w[q];
+      for (int q = 0; q < LA; q++) sa.a[q] = wrap_a ? nxt.a[q] : cur.a[q];
 #pragma unroll
-      for (int q = 0; q < 4; q++) src.a[q] = wrap ? nxt.a[q] : cur.a[q];
-      __builtin_amdgcn_sched_barrier(0);
-      // k-step 0 of the stage: its fragments are in set 0; read those of k-step 1, request half of stage g+3
-#pragma unroll
-      for (int m = 0; m < 16; m++) {
-        acc[m >> 2][m & 3] =
-            __builtin_amdgcn_mfma_f32_32x32x16_bf16(F[0][m >> 2], F[0][4 + (m & 3)], acc[m >> 2][m & 3], 0, 0, 0);
-        if (m < 8) rd(cb, 1, 1, RO[m]);
-        else if (m >= 10 && (m & 1) == 0) issue(src, s3, pb, (m - 10) >> 1);
-        __builtin_amdgcn_sched_barrier(0);
+      for (int q = 0; q < LW; q++) {
+        s0.w[q] = wrap_w0 ? nxt.w[q] : cur.w[q];
+        s1.w[q] = wrap_w1 ? nxt.w[q] : cur.w[q];
       }
-      // behind stage g+1 were issued stage g+2 (8 loads) and five loads of stage g+3
-      wait_vmcnt<TALL_LOADS + 5>();
+      const int ca = (wrap_a ? s + 4 - S : s + 4) >> 1;
+      const int sw0 = wrap_w0 ? s + 3 - S : s + 3, sw1 = wrap_w1 ? s + 4 - S : s + 4;
+      __builtin_amdgcn_sched_barrier(0);
+      // Every k-step issues a quarter of A chunk s / 2 + 2, into the buffer that chunk s / 2 - 1 left
+      // (every wave is past the barrier of the stage that read it last), and half of a W stage,
+      // behind the fragment reads: loads(x, ...) places them after MFMAs NR, NR + 2, ...
+      auto loads = [&](int m, int x, const TallSrc<SH> &sw_, int st, int wbuf, int half) {
+#pragma unroll
+        for (int q = 0; q < LA1; q++)
+          if (m == NR + 2 * q) issue_a(sa, ca, ab2, x * LA1 + q);
+#pragma unroll
+        for (int q = 0; q < LW1; q++)
+          if (m == NR + 2 * (LA1 + q)) issue_w(sw_, st, wbuf, half * LW1 + q);
+      };
+      kstep(0, g & 3, 1, ab, 1, [&](int m) { loads(m, 0, s0, sw0, (g + 3) & 3, 0); });
+      // behind W stage s+1 were issued the loads of two k-steps of stage s-1 and of one of stage s
+      wait_vmcnt<3 * (LA1 + LW1)>();
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       __builtin_amdgcn_s_barrier();
       __builtin_amdgcn_sched_barrier(0);
-      // k-step 1: read k-step 0 of the next stage, request the other half of stage g+3
-#pragma unroll
-      for (int m = 0; m < 16; m++) {
-        acc[m >> 2][m & 3] =
-            __builtin_amdgcn_mfma_f32_32x32x16_bf16(F[1][m >> 2], F[1][4 + (m & 3)], acc[m >> 2][m & 3], 0, 0, 0);
-        if (m < 8) rd(nb, 0, 0, RO[m]);
-        else if (m >= 10 && (m & 1) == 0) issue(src, s3, pb, 3 + ((m - 10) >> 1));
-        __builtin_amdgcn_sched_barrier(0);
-      }
+      kstep(1, (g + 1) & 3, 0, ab, 2, [&](int m) { loads(m, 1, s0, sw0, (g + 3) & 3, 1); });
+      // ---- odd stage s+1: the second half of the chunk -----------------------------------------
+      kstep(0, (g + 1) & 3, 1, ab, 3, [&](int m) { loads(m, 2, s1, sw1, (g + 4) & 3, 0); });
+      // W stage s+2, and with it the A chunk that the next stage starts (its last loads went out in
+      // front of that stage's), must have landed
+      wait_vmcnt<3 * (LA1 + LW1)>();
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+      kstep(1, (g + 2) & 3, 0, ab1, 0, [&](int m) { loads(m, 3, s1, sw1, (g + 4) & 3, 1); });
+      ab = ab1;
     }
-    // epilogue: the wave's four column blocks, each with its four 32-row blocks.  The empty asm pins
-    // a column block's accumulators in their AGPRs until the block before it has been stored: left
-    // alone, the compiler copies all 256 of them to VGPRs where the stage loop ends, and spills.
+    // epilogue: the wave's column blocks, each with its row blocks.  The empty asm pins a column
+    // block's accumulators in their AGPRs until the block before it has been stored: left alone,
+    // the compiler copies every accumulator to VGPRs where the stage loop ends, and spills.
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-      asm volatile("" : "+a"(acc[i][0]), "+a"(acc[i][1]), "+a"(acc[i][2]), "+a"(acc[i][3]));
-      const int n0 = cur.ct * TALL_BN + (wc * 4 + i) * 32;
-      if (n0 < N) epilogue_store<4, EPI, true>(p, cur.mat, cur.row0 + wr * 128, cur.rows - wr * 128, n0, lane, acc[i]);
+    for (int i = 0; i < CB; i++) {
+#pragma unroll
+      for (int r = 0; r < RB; r++) asm volatile("" : "+a"(acc[i][r]));
+      const int n0 = cur.ct * SH::BN + (wc * CB + i) * 32;
+      if (n0 < N)
+        epilogue_store<RB, EPI, true>(p, cur.mat, cur.row0 + wr * RB * 32, cur.rows - wr * RB * 32, n0, lane, acc[i]);
     }
     if (!more) break;
     j = jn;
@@ -262,7 +317,7 @@ __global__ __launch_bounds__(TALL_THREADS, 1) void tall_gemm_kernel(GemmParams p
   wait_vmcnt<0>();
 }
 
-template <bool GATHER, int EPI>
+template <class SH, bool GATHER, int EPI>
 static int launch_tall(const GemmParams &p, int max_tiles, hipStream_t s) {
   constexpr int MAX_DEV = 64;
   static std::mutex mu;
@@ -270,43 +325,54 @@ static int launch_tall(const GemmParams &p, int max_tiles, hipStream_t s) {
   int dev = 0;
   GPTOSS_HIP(hipGetDevice(&dev));
   GPTOSS_REQUIRE(dev >= 0 && dev < MAX_DEV, GPTOSS_ERR_STATE, "run_gemm: device ordinal %d outside 0..%d", dev, MAX_DEV - 1);
-  auto kern = tall_gemm_kernel<GATHER, EPI>;
-  const size_t smem = (size_t)TALL_NST * TALL_STAGE + TALL_BM * 4;
+  auto kern = tall_gemm_kernel<SH, GATHER, EPI>;
   {
     std::lock_guard<std::mutex> lock(mu);
     if (!raised[dev]) {
       GPTOSS_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                     (int)smem));
+                                     SH::SMEM));
       raised[dev] = true;
     }
   }
-  const int total = max_tiles * p.n_col_tiles;
+  GemmParams q = p;
+  q.n_col_tiles = cdiv(p.N, SH::BN);
+  const int total = max_tiles * q.n_col_tiles;
   int grid = ((total + 7) / 8) * 8;
   if (grid > 256) grid = 256;
   if (grid == 0) return GPTOSS_OK;
   {
     TraceScope ts(GATHER ? "gemm1_gather_swiglu" : "gemm_f32", s);
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(TALL_THREADS), smem, s, p);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(TALL_THREADS), SH::SMEM, s, q);
   }
   GPTOSS_LAUNCH_CHECK("tall_gemm_kernel");
   return GPTOSS_OK;
 }
 
+// The shape in use.  Tiles of 128 rows for the dense GEMMs of a decode step of 1024 rows (128 x 96,
+// 128, 160 and 192 columns, on an earlier form of this kernel with 32-k stages for both operands)
+// came out bit-identical as well, and 3-4 us ahead of the streaming kernels' 41-43 us on the two
+// projections of the 20B shape: a wave that owns 3 to 6 output blocks has 4 to 6 fragment reads per
+// k-step of 100-200 cycles and nothing else to run while they are on their way, so even without any
+// load or store such a launch takes 21-28 us where its MFMAs alone take 15.  Not worth a second
+// dispatch rule.
+using Tall256 = TallShape<2, 2, 4, 4>;   // 256 x 256
+
 bool gemm_tall_applies(const GemmParams &p, bool gather, int epi) {
   const bool kind = (gather && epi == EPI_SWIGLU) || (!gather && epi == EPI_F32);
-  return kind && !p.w_mxfp4 && p.K % TALL_BK == 0 && p.K >= 8 * TALL_BK && p.N % 32 == 0;
+  // whole A chunks of 64 k, and at least 8 stages: an item's first loads are requested during the
+  // last four stages of the item before it
+  return kind && !p.w_mxfp4 && p.K % (2 * TALL_BK) == 0 && p.K >= 8 * TALL_BK && p.N % 32 == 0;
 }
 
-// p.n_col_tiles must count 256-column tiles (it does: gemm_col_tiles); tiles of at most 256 rows
 int run_gemm_tall(const GemmParams &p, bool gather, int epi, int max_tiles, long long max_rows, hipStream_t s) {
   GPTOSS_REQUIRE(gemm_tall_applies(p, gather, epi), GPTOSS_ERR_DIM,
-                 "run_gemm: 256-row tiles need bf16 weights, K %% 32 == 0, K >= 256, N %% 32 == 0 and the gather+SwiGLU "
-                 "or plain fp32 form (gather=%d epi=%d N=%d K=%d)", (int)gather, epi, p.N, p.K);
+                 "run_gemm: 256-row tiles need bf16 weights, K %% 64 == 0, K >= 256, N %% 32 == 0 and the "
+                 "gather+SwiGLU or plain fp32 form (gather=%d epi=%d N=%d K=%d)", (int)gather, epi, p.N, p.K);
   // a row of A is addressed by a 32-bit byte offset
   GPTOSS_REQUIRE(max_rows * p.K * 2 < (1ll << 32), GPTOSS_ERR_DIM,
                  "run_gemm: 256-row tiles need rows x K below 2^31 elements (rows<=%lld K=%d)", max_rows, p.K);
-  if (gather) return launch_tall<true, EPI_SWIGLU>(p, max_tiles, s);
-  return launch_tall<false, EPI_F32>(p, max_tiles, s);
+  if (gather) return launch_tall<Tall256, true, EPI_SWIGLU>(p, max_tiles, s);
+  return launch_tall<Tall256, false, EPI_F32>(p, max_tiles, s);
 }
 
 }  // namespace gptoss
