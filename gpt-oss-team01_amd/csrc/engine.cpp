@@ -652,8 +652,8 @@ extern "C" int gptoss_engine_create(const gptoss_config *cfg, const float *host_
   if (flags & GPTOSS_ENGINE_LOGITS) {
     e->logits = b.alloc<float>((size_t)B * V);
   } else {
-    e->amax_val = b.alloc<float>((size_t)B * gemm_col_tiles(V));
-    e->amax_idx = b.alloc<int>((size_t)B * gemm_col_tiles(V));
+    e->amax_val = b.alloc<float>((size_t)B * gemm_argmax_tiles(V));
+    e->amax_idx = b.alloc<int>((size_t)B * gemm_argmax_tiles(V));
   }
   e->moe_ws_bytes = gptoss_moe_workspace_bytes(B, E, k, H, I);
   e->moe_ws = b.alloc<unsigned char>(e->moe_ws_bytes);
@@ -776,8 +776,9 @@ static int step_impl(gptoss_engine *e, const int *host_tokens, int pos, const in
   } else {
     // the classifier keeps only (max, column) per row and column tile; a small second stage picks
     // the row's arg-max (lowest column among equal maxima, run.cpp:739-750)
-    STEP(dense_gemm(e->t, e->unembedding, nullptr, nullptr, EPI_ARGMAX, B, V, H, s, e->amax_val, e->amax_idx));
-    STEP(run_argmax_tiles(e->amax_val, e->amax_idx, e->d_next, B, gemm_col_tiles(V), s));
+    int pairs = 0;
+    STEP(dense_gemm(e->t, e->unembedding, nullptr, nullptr, EPI_ARGMAX, B, V, H, s, e->amax_val, e->amax_idx, &pairs));
+    STEP(run_argmax_tiles(e->amax_val, e->amax_idx, e->d_next, B, pairs, s));
   }
   GPTOSS_HIP(hipMemcpyAsync(e->h_next, e->d_next, sizeof(int) * B, hipMemcpyDeviceToHost, s));
   GPTOSS_HIP(hipStreamSynchronize(s));
@@ -877,8 +878,9 @@ static int prefill_chunk(gptoss_engine *e, const int *host_tokens, int seq0, int
     STEP(dense_gemm(e->t, e->unembedding, nullptr, e->logits + (size_t)seq0 * V, EPI_F32, Bc, V, H, s));
     STEP(run_argmax(e->logits + (size_t)seq0 * V, e->d_next + seq0, Bc, V, s));
   } else {
-    STEP(dense_gemm(e->t, e->unembedding, nullptr, nullptr, EPI_ARGMAX, Bc, V, H, s, e->amax_val, e->amax_idx));
-    STEP(run_argmax_tiles(e->amax_val, e->amax_idx, e->d_next + seq0, Bc, gemm_col_tiles(V), s));
+    int pairs = 0;
+    STEP(dense_gemm(e->t, e->unembedding, nullptr, nullptr, EPI_ARGMAX, Bc, V, H, s, e->amax_val, e->amax_idx, &pairs));
+    STEP(run_argmax_tiles(e->amax_val, e->amax_idx, e->d_next + seq0, Bc, pairs, s));
   }
 #undef STEP
   return GPTOSS_OK;
@@ -987,8 +989,9 @@ static int step_rows(gptoss_engine *e, int n, const int *tok, const int *slot, c
       STEP(run_argmax(lg, e->d_next + j, 1, V, s));
     }
   } else {
-    STEP(dense_gemm(e->t, e->unembedding, nullptr, nullptr, EPI_ARGMAX, n_sample, V, H, s, e->amax_val, e->amax_idx));
-    STEP(run_argmax_tiles(e->amax_val, e->amax_idx, e->d_next, n_sample, gemm_col_tiles(V), s));
+    int pairs = 0;
+    STEP(dense_gemm(e->t, e->unembedding, nullptr, nullptr, EPI_ARGMAX, n_sample, V, H, s, e->amax_val, e->amax_idx, &pairs));
+    STEP(run_argmax_tiles(e->amax_val, e->amax_idx, e->d_next, n_sample, pairs, s));
   }
   GPTOSS_HIP(hipMemcpyAsync(e->h_next, e->d_next, sizeof(int) * n_sample, hipMemcpyDeviceToHost, s));
   GPTOSS_HIP(hipStreamSynchronize(s));

@@ -21,7 +21,8 @@ struct GemmParams {
   const float *bias;   // [n_mat, N] or nullptr
   void *out;           // EPI_F32: float [*, N]; EPI_SWIGLU: bf16 [*, N/2]; EPI_BF16: bf16 [*, N]
   float *amax_val;     // EPI_ARGMAX (dense only): per (row, column tile) the largest value ...
-  int *amax_idx;       // ... and the lowest column that holds it, [rows, n_col_tiles]
+  int *amax_idx;       // ... and the lowest column that holds it, [rows, n_col_tiles] (the 256-row
+                       // kernel: per (row, 128-column half of a tile), [rows, 2 n_col_tiles])
   const int *tiles;    // {n_tiles, (mat,row0,rows)*} or nullptr for a dense problem
   const int *xcd_bounds;  // 9 positions in the tile list (tile << 16 | 16-bit fraction) that cut the
                           // work into 8 parts of equal estimated cost, or nullptr: equal item counts.
@@ -40,7 +41,7 @@ struct GemmParams {
 int run_gemm(const GemmParams &p, bool gather, int epi, int rows_per_tile, int max_tiles,
              hipStream_t s);
 // gemm_tall.hip: tiles of 256 x 256 with both operands through LDS, for launches of thousands of rows,
-// bound by the matrix cores (bf16 weights; gather + SwiGLU or plain fp32 output).  max_rows bounds
+// bound by the matrix cores (bf16 weights; gather + SwiGLU, plain fp32 output, or the row arg-max).  max_rows bounds
 // the rows of A that the launch can address.
 bool gemm_tall_applies(const GemmParams &p, bool gather, int epi);
 int run_gemm_tall(const GemmParams &p, bool gather, int epi, int max_tiles, long long max_rows, hipStream_t s);
@@ -73,10 +74,13 @@ int run_norm_router(float *x, const float *residual, const float *weight, void *
                     const float *b_router, float *logits, int B, int H, int E, int k, float *topk_w, int *topk_i,
                     hipStream_t s);
 int moe_rows_per_tile(int B, int k, int E, bool mxfp4);
-// dense C = A . W^T (+ bias) with the epilogue `epi`; EPI_ARGMAX fills amax_val / amax_idx [B, gemm_col_tiles(N)]
+// dense C = A . W^T (+ bias) with the epilogue `epi`; EPI_ARGMAX fills amax_val / amax_idx [B, *amax_tiles]
+// EPI_ARGMAX: *amax_tiles (required) receives the number of (value, column) pairs written per row,
+// at most gemm_argmax_tiles(N), for run_argmax_tiles to finish
 int dense_gemm(const bf16_t *A, const bf16_t *W, const float *bias, void *out, int epi, int B, int N, int K,
-               hipStream_t s, float *amax_val = nullptr, int *amax_idx = nullptr);
+               hipStream_t s, float *amax_val = nullptr, int *amax_idx = nullptr, int *amax_tiles = nullptr);
 int gemm_col_tiles(int N);  // column tiles of one workgroup's width
+inline int gemm_argmax_tiles(int N) { return 2 * gemm_col_tiles(N); }  // pairs per row to allocate for EPI_ARGMAX
 // moe_route.hip
 int run_router(const void *t, const void *w_router, const float *b_router, float *logits, int B,
                int H, int E, int k, float *topk_w, int *topk_i, hipStream_t s);

@@ -301,13 +301,71 @@ __global__ __launch_bounds__(TALL_THREADS, 1) void tall_gemm_kernel(GemmParams p
     // epilogue: the wave's column blocks, each with its row blocks.  The empty asm pins a column
     // block's accumulators in their AGPRs until the block before it has been stored: left alone,
     // the compiler copies every accumulator to VGPRs where the stage loop ends, and spills.
+    if constexpr (EPI == EPI_ARGMAX) {
+      // Row-wise arg-max of the wave's CB x 32 columns without writing the products.  A lane holds
+      // one row of each row block and 16 channels of each column block: it scans them in ascending
+      // column order with a strict >, so the lowest column wins a tie; the two half-waves are merged
+      // with the same rule, and the first 32 lanes write the (value, column) pair of their rows for
+      // this half of the column tile.
+      float bv[RB];
+      int bi[RB];
 #pragma unroll
-    for (int i = 0; i < CB; i++) {
+      for (int r = 0; r < RB; r++) {
+        bv[r] = -INFINITY;
+        bi[r] = 0x7fffffff;
+      }
+      const const_as<float> bias = constant_ptr(p.bias);
 #pragma unroll
-      for (int r = 0; r < RB; r++) asm volatile("" : "+a"(acc[i][r]));
-      const int n0 = cur.ct * SH::BN + (wc * CB + i) * 32;
-      if (n0 < N)
-        epilogue_store<RB, EPI, true>(p, cur.mat, cur.row0 + wr * RB * 32, cur.rows - wr * RB * 32, n0, lane, acc[i]);
+      for (int i = 0; i < CB; i++) {
+#pragma unroll
+        for (int r = 0; r < RB; r++) asm volatile("" : "+a"(acc[i][r]));
+        const int n0 = cur.ct * SH::BN + (wc * CB + i) * 32;
+        if (n0 < N) {
+#pragma unroll
+          for (int gq = 0; gq < 16; gq++) {
+            const int c_lo = n0 + (gq >> 2) * 8 + (gq & 3), c_hi = c_lo + 4;
+            float b = 0.f;
+            if (p.bias) {
+              const float b_lo = bias[c_lo], b_hi = bias[c_hi];
+              b = h ? b_hi : b_lo;
+            }
+            const int col = h ? c_hi : c_lo;
+#pragma unroll
+            for (int r = 0; r < RB; r++) {
+              const float v = acc[i][r][gq] + b;
+              if (v > bv[r]) {
+                bv[r] = v;
+                bi[r] = col;
+              }
+            }
+          }
+        }
+      }
+#pragma unroll
+      for (int r = 0; r < RB; r++) {
+        const float ov = __shfl_xor(bv[r], 32, 64);
+        const int oi = __shfl_xor(bi[r], 32, 64);
+        if (ov > bv[r] || (ov == bv[r] && oi < bi[r])) {
+          bv[r] = ov;
+          bi[r] = oi;
+        }
+        const int row = (wr * RB + r) * 32 + lane;
+        if (lane < 32 && row < cur.rows) {
+          const size_t o = (size_t)(cur.row0 + row) * (SH::WC * p.n_col_tiles) + cur.ct * SH::WC + wc;
+          p.amax_val[o] = bv[r];
+          p.amax_idx[o] = bi[r];
+        }
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < CB; i++) {
+#pragma unroll
+        for (int r = 0; r < RB; r++) asm volatile("" : "+a"(acc[i][r]));
+        const int n0 = cur.ct * SH::BN + (wc * CB + i) * 32;
+        if (n0 < N)
+          epilogue_store<RB, EPI, true>(p, cur.mat, cur.row0 + wr * RB * 32, cur.rows - wr * RB * 32, n0, lane,
+                                        acc[i]);
+      }
     }
     if (!more) break;
     j = jn;
@@ -341,7 +399,7 @@ static int launch_tall(const GemmParams &p, int max_tiles, hipStream_t s) {
   if (grid > 256) grid = 256;
   if (grid == 0) return GPTOSS_OK;
   {
-    TraceScope ts(GATHER ? "gemm1_gather_swiglu" : "gemm_f32", s);
+    TraceScope ts(EPI == EPI_ARGMAX ? "gemm_argmax" : GATHER ? "gemm1_gather_swiglu" : "gemm_f32", s);
     hipLaunchKernelGGL(kern, dim3(grid), dim3(TALL_THREADS), SH::SMEM, s, q);
   }
   GPTOSS_LAUNCH_CHECK("tall_gemm_kernel");
@@ -358,7 +416,8 @@ static int launch_tall(const GemmParams &p, int max_tiles, hipStream_t s) {
 using Tall256 = TallShape<2, 2, 4, 4>;   // 256 x 256
 
 bool gemm_tall_applies(const GemmParams &p, bool gather, int epi) {
-  const bool kind = (gather && epi == EPI_SWIGLU) || (!gather && epi == EPI_F32);
+  const bool kind = (gather && epi == EPI_SWIGLU) || (!gather && epi == EPI_F32) ||
+                    (!gather && epi == EPI_ARGMAX && p.tiles == nullptr && p.amax_val && p.amax_idx);
   // whole A chunks of 64 k, and at least 8 stages: an item's first loads are requested during the
   // last four stages of the item before it
   return kind && !p.w_mxfp4 && p.K % (2 * TALL_BK) == 0 && p.K >= 8 * TALL_BK && p.N % 32 == 0;
@@ -367,10 +426,12 @@ bool gemm_tall_applies(const GemmParams &p, bool gather, int epi) {
 int run_gemm_tall(const GemmParams &p, bool gather, int epi, int max_tiles, long long max_rows, hipStream_t s) {
   GPTOSS_REQUIRE(gemm_tall_applies(p, gather, epi), GPTOSS_ERR_DIM,
                  "run_gemm: 256-row tiles need bf16 weights, K %% 64 == 0, K >= 256, N %% 32 == 0 and the "
-                 "gather+SwiGLU or plain fp32 form (gather=%d epi=%d N=%d K=%d)", (int)gather, epi, p.N, p.K);
+                 "gather+SwiGLU, plain fp32 or dense arg-max form (gather=%d epi=%d N=%d K=%d)", (int)gather, epi, p.N, p.K);
   // a row of A is addressed by a 32-bit byte offset
   GPTOSS_REQUIRE(max_rows * p.K * 2 < (1ll << 32), GPTOSS_ERR_DIM,
                  "run_gemm: 256-row tiles need rows x K below 2^31 elements (rows<=%lld K=%d)", max_rows, p.K);
+  static_assert(Tall256::WC == 2, "dense_gemm reports two arg-max pairs per row and column tile");
+  if (epi == EPI_ARGMAX) return launch_tall<Tall256, false, EPI_ARGMAX>(p, max_tiles, s);
   if (gather) return launch_tall<Tall256, true, EPI_SWIGLU>(p, max_tiles, s);
   return launch_tall<Tall256, false, EPI_F32>(p, max_tiles, s);
 }

@@ -41,7 +41,7 @@ extern "C" int gptoss_dense_gemm(const void *a, const void *w_packed, const floa
 
 extern "C" size_t gptoss_classifier_argmax_workspace_bytes(int B, int V) {
   if (B <= 0 || V <= 0) return 0;
-  return 2 * align_up((size_t)B * gemm_col_tiles(V) * sizeof(float), 256);
+  return 2 * align_up((size_t)B * gemm_argmax_tiles(V) * sizeof(float), 256);
 }
 
 extern "C" int gptoss_classifier_argmax(const void *a, const void *w_packed, int *next_ids, int B, int V, int K,
@@ -50,15 +50,16 @@ extern "C" int gptoss_classifier_argmax(const void *a, const void *w_packed, int
   if (rc != GPTOSS_OK) return rc;
   GPTOSS_REQUIRE(next_ids, GPTOSS_ERR_NULL, "classifier_argmax: null pointer");
   if (B == 0) return GPTOSS_OK;
-  const size_t half = align_up((size_t)B * gemm_col_tiles(V) * sizeof(float), 256);
+  const size_t half = align_up((size_t)B * gemm_argmax_tiles(V) * sizeof(float), 256);
   GPTOSS_REQUIRE(workspace && aligned(workspace, 256) && workspace_bytes >= 2 * half, GPTOSS_ERR_WORKSPACE,
                  "classifier_argmax: workspace missing, misaligned or smaller than %zu bytes", 2 * half);
   float *val = (float *)workspace;
   int *idx = (int *)((unsigned char *)workspace + half);
+  int pairs = 0;
   rc = dense_gemm((const bf16_t *)a, (const bf16_t *)w_packed, nullptr, nullptr, EPI_ARGMAX, B, V, K,
-                  (hipStream_t)stream, val, idx);
+                  (hipStream_t)stream, val, idx, &pairs);
   if (rc != GPTOSS_OK) return rc;
-  return run_argmax_tiles(val, idx, next_ids, B, gemm_col_tiles(V), (hipStream_t)stream);
+  return run_argmax_tiles(val, idx, next_ids, B, pairs, (hipStream_t)stream);
 }
 
 extern "C" int gptoss_argmax(const float *logits, int *ids, int B, int V, void *stream) {

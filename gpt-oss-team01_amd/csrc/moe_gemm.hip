@@ -274,10 +274,21 @@ static int dense_tall_min_rows() {
   return v;
 }
 
+// rows from which the classifier's arg-max GEMM uses it (measured, vocabulary 201088 x 2880: 256 rows
+// 360 -> 295 us, 512 rows 716 -> 556, 1024 rows 1194 -> 986-1007, 2048 rows 2319 -> 1859)
+static int argmax_tall_min_rows() {
+  static const int v = [] {
+    const char *e = getenv("GPTOSS_ARGMAX_TALL_MIN_ROWS");
+    const int n = e ? atoi(e) : 0;
+    return n > 0 ? n : 256;
+  }();
+  return v;
+}
+
 // C[B, N] = A[B, K] . W[N, K]^T (+ bias): the dense GEMMs of a step (QKV and output projections,
 // classifier), with the kernel and row tile chosen from the batch size.
 int dense_gemm(const bf16_t *A, const bf16_t *W, const float *bias, void *out, int epi, int B, int N,
-               int K, hipStream_t s, float *amax_val, int *amax_idx) {
+               int K, hipStream_t s, float *amax_val, int *amax_idx, int *amax_tiles) {
   GemmParams g{};
   g.amax_val = amax_val;
   g.amax_idx = amax_idx;
@@ -318,7 +329,12 @@ int dense_gemm(const bf16_t *A, const bf16_t *W, const float *bias, void *out, i
       }
     }
   }
-  if (B >= dense_tall_min_rows() && gemm_tall_applies(g, false, epi)) rpt = 256;
+  if (B >= (epi == EPI_ARGMAX ? argmax_tall_min_rows() : dense_tall_min_rows()) && gemm_tall_applies(g, false, epi))
+    rpt = 256;
+  if (epi == EPI_ARGMAX) {
+    GPTOSS_REQUIRE(amax_tiles, GPTOSS_ERR_NULL, "dense_gemm: the arg-max form reports its pairs per row");
+    *amax_tiles = rpt == 256 ? 2 * g.n_col_tiles : g.n_col_tiles;
+  }
   return run_gemm(g, false, epi, rpt, cdiv(B, rpt), s);
 }
 

@@ -70,7 +70,8 @@ def test_dense_gemm_of_a_prompt_pass_equals_the_same_rows_in_small_batches(ops, 
         assert torch.equal(full[r0:r0 + step], ops.dense_gemm(a[r0:r0 + step].contiguous(), wp, N, b)), r0
 
 
-@pytest.mark.parametrize("B,V,K", [(5, 4096, 256), (130, 201088, 2880), (1024, 50304, 512), (515, 9984, 256)])
+@pytest.mark.parametrize("B,V,K", [(5, 4096, 256), (130, 201088, 2880), (1024, 50304, 512), (515, 9984, 256),
+                                   (256, 9984, 512), (255, 4128, 320)])
 def test_classifier_argmax_equals_argmax_of_logits(ops, B, V, K):
     g = torch.Generator(device="cuda").manual_seed(V)
     a = torch.randn(B, K, device="cuda", generator=g).to(torch.bfloat16)
@@ -81,6 +82,26 @@ def test_classifier_argmax_equals_argmax_of_logits(ops, B, V, K):
     ids = ops.classifier_argmax(a, wp, V).cpu().numpy()
     assert np.array_equal(ids, logits.cpu().numpy().argmax(axis=1))
     assert np.array_equal(ops.argmax(logits).cpu().numpy(), ids)
+
+
+@pytest.mark.parametrize("B", [130, 600])
+@pytest.mark.parametrize("cols", [(7, 11, 40, 135, 300, 4127), (11, 40, 135), (135, 300), (200, 250), (259, 263)])
+def test_classifier_argmax_ties_pick_the_lowest_column(ops, B, cols):
+    """Equal maxima in the two half-waves of a lane pair, in two column blocks of a wave, in the two
+    waves that share a row, in two column tiles and in the last, partly filled tile: the lowest
+    column wins (run.cpp:739-750), on the streaming kernel (130 rows) and the 256-row kernel (600)."""
+    V, K = 4128, 256
+    g = torch.Generator(device="cuda").manual_seed(B)
+    a = torch.randn(B, K, device="cuda", generator=g).to(torch.bfloat16)
+    w = (torch.randn(V, K, device="cuda", generator=g) * 0.05).to(torch.bfloat16)
+    big = (w[cols[0]].float() * 8).to(torch.bfloat16)
+    for c in cols:
+        w[c] = big
+    ids = ops.classifier_argmax(a, ops.pack_weight(w), V).cpu().numpy()
+    logits = (a.float() @ w.float().T).cpu().numpy()
+    wins = logits[:, cols[0]] >= logits.max(axis=1)               # rows where the repeated column is the maximum
+    assert wins.sum() > B // 10
+    assert (ids[wins] == min(cols)).all()
 
 
 def test_argmax_ties_lowest_index(ops):
