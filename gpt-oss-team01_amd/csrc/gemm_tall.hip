@@ -411,8 +411,9 @@ static int launch_tall(const GemmParams &p, int max_tiles, hipStream_t s) {
 // came out bit-identical as well, and 3-4 us ahead of the streaming kernels' 41-43 us on the two
 // projections of the 20B shape: a wave that owns 3 to 6 output blocks has 4 to 6 fragment reads per
 // k-step of 100-200 cycles and nothing else to run while they are on their way, so even without any
-// load or store such a launch takes 21-28 us where its MFMAs alone take 15.  Not worth a second
-// dispatch rule.
+// load or store such a launch takes 21-28 us where its MFMAs alone take 15.  128 x 128 tiles with two
+// workgroups per CU (80 KB of LDS each, on this form of the kernel) did not move that either: 48 and
+// 41 us against 43 and 43.  Not worth a second dispatch rule.
 using Tall256 = TallShape<2, 2, 4, 4>;   // 256 x 256
 
 bool gemm_tall_applies(const GemmParams &p, bool gather, int epi) {
