@@ -259,8 +259,9 @@ int gptoss_dense_gemm(const void *a, const void *w_packed, const float *bias, fl
                       int K, void *stream);
 
 /* next_ids[b] = arg max over v of a[b,:] . w[v,:]  (lowest v among equal maxima) without writing the
- * [B,V] logits: the classifier GEMM keeps (max, column) per row and 256-column tile, a second small
- * kernel picks the row's winner.  Replaces classifier_gemm_batched_v2_quantize + max_logits_batched
+ * [B,V] logits: the classifier GEMM keeps (max, column) per row and 256-column tile (per 128-column
+ * half of a tile from 256 rows on, where it runs on 256-row tiles), a second small kernel picks the
+ * row's winner.  Replaces classifier_gemm_batched_v2_quantize + max_logits_batched
  * (layer_hip_batch.cpp:1465-1501, 1542-1630; model.cpp:144-148). */
 size_t gptoss_classifier_argmax_workspace_bytes(int B, int V);
 int gptoss_classifier_argmax(const void *a, const void *w_packed, int *next_ids, int B, int V, int K,
