@@ -527,7 +527,7 @@ __global__ __launch_bounds__(GEMM_THREADS, (gemm_two_per_cu(MBMAX, FP4) ? 4 : 2)
 
   struct Item {
     int mat, row0, rows, ct;
-    bool once;  // no other row tile multiplies this item's W
+    int once;  // no other row tile multiplies this item's W (an int: the struct has no padding to copy)
   };
   auto decode = [&](int jj) {
     const int work = lo + jj;
