@@ -20,7 +20,9 @@
 // behind the one waited for; stores of the previous item's epilogue that are still in flight only
 // make a wait stricter).
 // Same operand roles (W fragment first: lane = token row, registers = channels), same k order and
-// the same epilogue code as gemm_kernel.hpp, so the results are bit-identical to it.
+// the same epilogue code as gemm_kernel.hpp, so the results are bit-identical to it.  Three forms:
+// gather + SwiGLU (GEMM1 of a prompt pass), plain fp32 output (GEMM2, the projections), and the row
+// arg-max of the classifier, which writes no products at all and is the fastest of the three.
 #include <mutex>
 
 #include "gemm_kernel.hpp"
