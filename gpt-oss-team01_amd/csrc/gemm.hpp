@@ -44,6 +44,11 @@ int run_gemm(const GemmParams &p, bool gather, int epi, int rows_per_tile, int m
 // bound by the matrix cores (bf16 weights; gather + SwiGLU, plain fp32 output, or the row arg-max).  max_rows bounds
 // the rows of A that the launch can address.
 bool gemm_tall_applies(const GemmParams &p, bool gather, int epi);
+// what the 256-row kernels need of a problem besides its form: whole 64-k chunks, at least 8 stages
+// of 32 k, whole 32-column blocks, and every row of A within a 32-bit byte offset
+inline bool gemm_tall_shape_ok(int N, int K, long long max_rows) {
+  return K % 64 == 0 && K >= 256 && N % 32 == 0 && max_rows * K * 2 < (1ll << 32);
+}
 int run_gemm_tall(const GemmParams &p, bool gather, int epi, int max_tiles, long long max_rows, hipStream_t s);
 // norm_w / norm_out (optional, accumulate only): also write RMSNorm(out) * norm_w as bf16.  Returns
 // with only the combine done when the fused form does not apply (H > 4096 or misaligned); the

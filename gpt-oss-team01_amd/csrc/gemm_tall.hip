@@ -423,7 +423,8 @@ bool gemm_tall_applies(const GemmParams &p, bool gather, int epi) {
                     (!gather && epi == EPI_ARGMAX && p.tiles == nullptr && p.amax_val && p.amax_idx);
   // whole A chunks of 64 k, and at least 8 stages: an item's first loads are requested during the
   // last four stages of the item before it
-  return kind && !p.w_mxfp4 && p.K % (2 * TALL_BK) == 0 && p.K >= 8 * TALL_BK && p.N % 32 == 0;
+  static_assert(2 * TALL_BK == 64, "gemm_tall_shape_ok states the chunk size");
+  return kind && !p.w_mxfp4 && gemm_tall_shape_ok(p.N, p.K, 0);
 }
 
 int run_gemm_tall(const GemmParams &p, bool gather, int epi, int max_tiles, long long max_rows, hipStream_t s) {

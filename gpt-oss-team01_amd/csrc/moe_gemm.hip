@@ -329,7 +329,8 @@ int dense_gemm(const bf16_t *A, const bf16_t *W, const float *bias, void *out, i
       }
     }
   }
-  if (B >= (epi == EPI_ARGMAX ? argmax_tall_min_rows() : dense_tall_min_rows()) && gemm_tall_applies(g, false, epi))
+  if (B >= (epi == EPI_ARGMAX ? argmax_tall_min_rows() : dense_tall_min_rows()) && gemm_tall_applies(g, false, epi) &&
+      gemm_tall_shape_ok(N, K, B))
     rpt = 256;
   if (epi == EPI_ARGMAX) {
     GPTOSS_REQUIRE(amax_tiles, GPTOSS_ERR_NULL, "dense_gemm: the arg-max form reports its pairs per row");

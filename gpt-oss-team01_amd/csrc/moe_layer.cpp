@@ -146,8 +146,10 @@ static int moe_forward_impl(const gptoss_moe_weights *w, const void *t, int B, f
   MoeWorkspace ws = carve(workspace, B, E, k, H, I);
   int rpt = moe_rows_per_tile(B, k, E, mxfp4 != 0);
   // a prompt pass, hundreds of rows per expert: bound by the matrix cores, not by streaming W
-  if (!mxfp4 && (long long)B * k >= (long long)moe_tall_min_rows() * E && H % 32 == 0 && H >= 256 && I % 32 == 0 &&
-      I >= 256)
+  // (the kernels address a row of A by a 32-bit byte offset: batches beyond that stay on the streaming kernels)
+  const long long tall_rows = ((long long)B * k / 256 + E) * 256;
+  if (!mxfp4 && (long long)B * k >= (long long)moe_tall_min_rows() * E && gemm_tall_shape_ok(2 * I, H, tall_rows) &&
+      gemm_tall_shape_ok(H, I, tall_rows))
     rpt = 256;
   const int max_tiles = gptoss_moe_max_tiles(B, k, E, rpt);
   // Each expert's row tiles are walked in blocks of up to MOE_TILE_BLOCK, column tile by column

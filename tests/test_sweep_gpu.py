@@ -139,18 +139,25 @@ def _engine_case(ops, orc, binfmt, D, nq, nkv, H, E, k, I, L, V, win, B, T, seed
         # unless, on the positions where the orders differ, the staged CPU model shows a router
         # decision of that row close enough to fall the other way.
         per = np.abs(lb - got).max(axis=1) / np.abs(got).max(axis=1)
-        assert np.median(per) <= 5e-3, (per, cfg)
-        for r in np.nonzero(per > TOL_MAX)[0]:
+        tie = {}
+        for r in np.nonzero(per > 5e-3)[0]:
             m = orc.Model(cfg, flat, stage=orc.STAGE_GPU)
             gaps = []
             for pos in range(T):
                 m.forward(int(toks[r, pos]), pos)
                 gaps.append(m.last_router_gap())
             m.close()
-            tie = min(gaps[win:])
-            assert tie < ROUTER_NEAR_TIE, ("prompt pass row beyond bf16 tolerance without a router near-tie",
-                                           int(r), float(per[r]), tie, cfg)
-            excused.append((int(r), float(per[r]), float(tie), win + int(np.argmin(gaps[win:]))))
+            tie[int(r)] = (float(min(gaps[win:])), win + int(np.argmin(gaps[win:])))
+        # rows without a near-tie stay tight (a near-tie that falls the same way still moves a row by
+        # up to a percent: one expert's weight shifts); rows beyond the bound must have one
+        clear = [r for r in range(B) if r not in tie or tie[r][0] >= ROUTER_NEAR_TIE]
+        if clear:
+            assert np.median(per[clear]) <= 5e-3, (per, cfg)
+        for r in range(B):
+            if per[r] > TOL_MAX:
+                assert r in tie and tie[r][0] < ROUTER_NEAR_TIE, (
+                    "prompt pass row beyond bf16 tolerance without a router near-tie", r, float(per[r]), tie.get(r), cfg)
+                excused.append((r, float(per[r]), tie[r][0], tie[r][1]))
         assert len(excused) <= max(1, B // 8), (excused, cfg)
     posv = np.array([T - (i % 2) for i in range(B)], np.int32)   # every other row repeats its last position
     a.step_ragged(np.array([toks[i, posv[i]] for i in range(B)], np.int32), posv)
@@ -210,3 +217,14 @@ def test_prompt_pass_past_the_window_differs_from_lock_step_only_at_router_near_
                               B=33, T=70, seed=355231429, tok_cols=72)
     print("rows excused by a router near-tie (row, max-rel, gap, position):", excused)
     assert [e[0] for e in excused] in ([19], []), excused
+
+
+def test_prompt_pass_of_a_single_row_with_a_near_tie_below_the_bound(ops, orc, binfmt):
+    """Another case of a long run: ONE sequence, 100-token prompt, window 64, three blocks, top-4 of 32
+    experts.  Its logits after the prompt pass differ from the lock-step ones by 1.7e-2 of their
+    scale, inside the bf16 bound but far above what rows without a close router decision show (a
+    median over one row is that row).  The staged CPU model puts two router scores 2.7e-4 apart at
+    position 90, past the ring: the row is counted as a near-tie row, not as a loose one."""
+    _, excused = _engine_case(ops, orc, binfmt, D=64, nq=2, nkv=2, H=256, E=32, k=4, I=128, L=3, V=4096, win=64,
+                              B=1, T=100, seed=480297126, tok_cols=102)
+    assert excused == []
