@@ -589,7 +589,7 @@ __global__ __launch_bounds__(GEMM_THREADS, (gemm_two_per_cu(MBMAX, FP4) ? 4 : 2)
       constexpr int M = decltype(m)::value;
       if (!done && (mb == M || M == MBMAX)) {
         // the refill of the ring from the next item follows this item's choice
-        if (cur.once)
+        if (!FP4 && cur.once)   // MXFP4 weights: a quarter of the bytes, not bound by their stream; one path keeps the 128-register kernels free of spills
           gemm_tile<M, MBMAX, NRING, GATHER, EPI, FP4, true>(p, lds, cur.mat, cur.row0, cur.rows, cur.ct, ring,
                                                              cur_w, nxt_w);
         else
