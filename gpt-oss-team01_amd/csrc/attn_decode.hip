@@ -610,9 +610,14 @@ __global__ __launch_bounds__(TILE_WAVES * 64, 4) void attn_prefill_tile_kernel(A
       stage[i] = *reinterpret_cast<const u32x4 *>(src + (size_t)(i * TILE_WAVES * 64 + tid) * 16);
   };
   auto store_block = [&](int buf) {
+    // the destination is recomputed at every block from a thread id the optimiser cannot see through:
+    // hoisted out of the loop it costs a register that the 128-register budget of two workgroups per
+    // CU does not have, and a spilled register's reload in the loop waits for the block in flight
+    int t_opaque = tid;
+    asm volatile("" : "+v"(t_opaque));
 #pragma unroll
     for (int i = 0; i < PASSES; i++) {
-      const int piece = i * TILE_WAVES * 64 + tid;
+      const int piece = i * TILE_WAVES * 64 + t_opaque;
       int dst = piece * 16;
       if (piece * 16 < K_BYTES) {
         const int r = piece / ROW_CHUNKS, j = piece % ROW_CHUNKS;
