@@ -48,11 +48,12 @@ static MoeWorkspace carve(void *base, int B, int E, int k, int H, int I) {
 // bf16 weights (32, 64, 128 or 160 rows): the smallest tile that holds an average expert's rows
 // plus 2.5 standard deviations of a uniform routing, so that nearly every expert is a single tile
 // and its weights are streamed exactly once; the kernel is bound by that stream.
-// MXFP4 weights (32, 64 or 96 rows): tiles of at most 96 rows, whose kernels run two workgroups
-// per CU; an expert's few row tiles are walked column tile by column tile (tile_block), so its
-// weights still come from HBM once.  96 rows only where they hold a whole expert; beyond that 64
-// (the 64-row kernel has room for a five-slab W ring, the 96-row one spills a few registers:
-// prompt passes of 8192 tokens 1.3 % faster with 64).
+// MXFP4 weights (32 or 64 rows): tiles of at most 64 rows, whose kernels run two workgroups per
+// CU within 128 registers; an expert's few row tiles are walked column tile by column tile
+// (tile_block), so its weights still come from HBM once.  The 96-row kernel does not fit that
+// budget (it spills 12-97 registers, and every reload in its slab loop waits for the loads in
+// flight): 384 / 512 tokens on 32 experts, where 96 rows would hold a whole expert, GEMM1 108 /
+// 119 us and GEMM2 141 / 150 us with it against 91 / 115 and 56 / 78 us with 64-row tiles.
 static int env_int(const char *name, int dflt) {
   const char *e = getenv(name);
   const int n = e ? atoi(e) : 0;
@@ -70,9 +71,7 @@ int moe_rows_per_tile(int B, int k, int E, bool mxfp4) {
 
   if (need <= 32) return 32;
   if (need <= 64) return 64;
-  if (mxfp4) {
-    return need <= 96 ? 96 : 64;
-  }
+  if (mxfp4) return 64;
   if (need <= 128) return 128;
   return 160;
 }

@@ -24,8 +24,9 @@ def _dequant(orc, blocks, scales):
 
 
 # token counts chosen to reach every row-tile size of the MXFP4 policy: 32 rows (200 tokens over 128
-# experts), 64 (64 and 300 tokens over 8), 96 (130 tokens over 8: 65 rows per expert) and 64 with
-# several tiles per expert (520 tokens over 8); the bf16 layer it is compared with uses 128/160 rows
+# experts), 64 (64 and 300 tokens over 8), 64 with two tiles for most experts (130 tokens over 8: 65
+# rows per expert) and with several (520 tokens over 8); the bf16 layer it is compared with uses
+# 128/160 rows
 @pytest.mark.parametrize("B,E,H,I,skew", [(64, 8, 256, 256, False), (300, 8, 256, 512, True),
                                           (200, 128, 2880, 2880, True), (130, 8, 256, 256, False),
                                           (520, 8, 512, 256, True)])
