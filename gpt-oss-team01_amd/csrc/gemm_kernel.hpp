@@ -38,6 +38,7 @@ constexpr int GEMM_THREADS = GEMM_WAVES * 64;
 constexpr int BK = 64;            // k per LDS slab (4 MFMA k-steps)
 constexpr int LDS_ROW = BK + 8;   // padded row length in bf16 elements (144 B)
 constexpr int BN = GEMM_WAVES * 32;  // columns per workgroup
+constexpr int HOLD_ROW = BN / 2 + 8;  // row of a SwiGLU output tile that waits in LDS: 128 outputs + padding (272 B)
 
 // MXFP4 operand expansion.  One dword holds the lane's 8 e2m1 codes of a k-step in checkpoint
 // order (byte j = elements 2j in the low and 2j+1 in the high nibble), which is what the hardware
@@ -134,9 +135,12 @@ __device__ __forceinline__ void w_load(WRing<NRING, FP4> &ring, const WStream &s
 // do not queue behind the vector loads already in flight for the next item.
 // CONST_BIAS: read the biases through the constant address space, for a kernel whose asm statements
 // would otherwise turn these loads into vector loads.
+// hold != nullptr (SwiGLU form only): the tile goes to LDS instead of memory, row r of the tile at
+// hold + r * HOLD_ROW, this wave's 16 outputs from column hold_col on.
 template <int MB, int EPI, bool CONST_BIAS = false>
 __device__ __forceinline__ void epilogue_store(const GemmParams &p, int mat, int row0, int rows, int n0,
-                                               int lane, const f32x16 (&acc)[MB]) {
+                                               int lane, const f32x16 (&acc)[MB], bf16_t *hold = nullptr,
+                                               int hold_col = 0) {
   const int N = p.N;
   const int tok = lane & 31;
   const bool hi = lane >= 32;
@@ -181,8 +185,9 @@ __device__ __forceinline__ void epilogue_store(const GemmParams &p, int mat, int
             const float e = __builtin_amdgcn_exp2f(-1.702f * 1.4426950408889634f * gate);
             v[q] = gate * __builtin_amdgcn_rcpf(1.0f + e) * (up + 1.0f);
           }
-          *reinterpret_cast<u32x2 *>(orow + lane_off + g * 8) =
-              u32x2{pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+          const u32x2 pk = u32x2{pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+          if (hold) *reinterpret_cast<u32x2 *>(hold + (i * 32 + tok) * HOLD_ROW + hold_col + h4 + g * 8) = pk;
+          else *reinterpret_cast<u32x2 *>(orow + lane_off + g * 8) = pk;
         }
       }
     }
@@ -226,7 +231,7 @@ __device__ __forceinline__ void epilogue_store(const GemmParams &p, int mat, int
 template <int MB, int MBMAX, int NRING, bool GATHER, int EPI, bool FP4, bool ONCE>
 __device__ __forceinline__ void gemm_tile(const GemmParams &p, bf16_t *lds, int mat, int row0, int rows,
                                           int ct, WRing<NRING, FP4> &ring, const WStream &cur,
-                                          const WStream &next) {
+                                          const WStream &next, bf16_t *hold = nullptr) {
   constexpr int LDS_STAGE = MBMAX * 32 * LDS_ROW;  // elements per A stage
   constexpr int D = NRING - 1;                     // slabs of W in flight
   constexpr int BQ = WRing<NRING, FP4>::BQ;
@@ -473,8 +478,13 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, bf16_t *lds, int 
   }
   if (!wave_active) return;
 
-  epilogue_store<MB, EPI>(p, mat, row0, rows, n0, lane, acc);
+  epilogue_store<MB, EPI>(p, mat, row0, rows, n0, lane, acc, hold, wave * 16);
 }
+
+// Kernels that keep two finished SwiGLU tiles in LDS until the workgroup's last item is done (see
+// grouped_gemm_kernel): GEMM1 with bf16 weights, whose bf16 tile of up to 160 x 128 outputs fits twice
+// behind the A stages of one workgroup per CU (156 KB at 160 rows).
+constexpr bool gemm_holds_output(bool gather, int epi, bool fp4) { return gather && epi == EPI_SWIGLU && !fp4; }
 
 // NRING: slabs of W held in registers per wave, NRING-1 of them in flight.  Three everywhere
 // except the 64-row MXFP4 kernels, where a slab costs 5 registers and two more ring slots fit under
@@ -503,7 +513,7 @@ __global__ __launch_bounds__(GEMM_THREADS, (gemm_two_per_cu(MBMAX, FP4) ? 4 : 2)
   constexpr int BM = MBMAX * 32;
   constexpr int NRING = gemm_nring(MBMAX, FP4);
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-  bf16_t *lds = reinterpret_cast<bf16_t *>(smem_raw);  // [3][BM][LDS_ROW]
+  bf16_t *lds = reinterpret_cast<bf16_t *>(smem_raw);  // [3][BM][LDS_ROW], then [2][BM][HOLD_ROW] where outputs are held
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
 
@@ -570,6 +580,18 @@ __global__ __launch_bounds__(GEMM_THREADS, (gemm_two_per_cu(MBMAX, FP4) ? 4 : 2)
     return it;
   };
 
+  // bf16 GEMM1: the outputs of the two work items before a workgroup's last one wait in LDS (behind
+  // the A stages) and are written after the last item's.  Output lines that turn dirty in L2 while
+  // the other workgroups still stream W are written back in the middle of that stream, and the
+  // write-backs slow the reads far beyond their share of the bytes: with three items per workgroup
+  // (the 1024-token layer) the slab loops of the second and third item take 60-65 us where the first
+  // item's takes 52, and 47-50 us without the stores.  Held back, the 23 MB leave the chip when the
+  // reads are over: GEMM1 213 -> 203 us, the layer 0.386 -> 0.375 ms on the same box.
+  constexpr bool HOLD = gemm_holds_output(GATHER, EPI, FP4);
+  bf16_t *hold_base = lds + 3 * BM * LDS_ROW;
+  const int n_mine = (hi - lo - j + per_xcd - 1) / per_xcd;
+  int it = 0;
+  int held_row0_a = 0, held_rows_a = 0, held_ct_a = 0, held_row0_b = 0, held_rows_b = 0, held_ct_b = 0;
   Item cur = decode(j);
   WStream cur_w = w_stream<FP4>(p, cur.mat, cur.ct, wave);
   WRing<NRING, FP4> ring;
@@ -584,6 +606,20 @@ __global__ __launch_bounds__(GEMM_THREADS, (gemm_two_per_cu(MBMAX, FP4) ? 4 : 2)
     const WStream nxt_w = more ? w_stream<FP4>(p, nxt.mat, nxt.ct, wave) : cur_w;
     // one fully unrolled code path per number of 32-row blocks actually present in the tile
     const int mb = (cur.rows + 31) >> 5;
+    bf16_t *hold_ptr = nullptr;
+    if (HOLD && it >= n_mine - 3 && it < n_mine - 1) {
+      const int slot = it & 1;
+      hold_ptr = hold_base + slot * (BM * HOLD_ROW);
+      if (slot == 0) {
+        held_row0_a = cur.row0;
+        held_rows_a = cur.rows;
+        held_ct_a = cur.ct;
+      } else {
+        held_row0_b = cur.row0;
+        held_rows_b = cur.rows;
+        held_ct_b = cur.ct;
+      }
+    }
     bool done = false;
     static_for<1, MBMAX + 1>([&](auto m) {
       constexpr int M = decltype(m)::value;
@@ -591,25 +627,42 @@ __global__ __launch_bounds__(GEMM_THREADS, (gemm_two_per_cu(MBMAX, FP4) ? 4 : 2)
         // the refill of the ring from the next item follows this item's choice
         if (!FP4 && cur.once)   // MXFP4 weights: a quarter of the bytes, not bound by their stream; one path keeps the 128-register kernels free of spills
           gemm_tile<M, MBMAX, NRING, GATHER, EPI, FP4, true>(p, lds, cur.mat, cur.row0, cur.rows, cur.ct, ring,
-                                                             cur_w, nxt_w);
+                                                             cur_w, nxt_w, hold_ptr);
         else
           gemm_tile<M, MBMAX, NRING, GATHER, EPI, FP4, false>(p, lds, cur.mat, cur.row0, cur.rows, cur.ct, ring,
-                                                              cur_w, nxt_w);
+                                                              cur_w, nxt_w, hold_ptr);
         done = true;
       }
     });
     if (!more) break;
     // every wave must be done reading this item's last A slab before the next prologue overwrites it
     __syncthreads();
+    it++;
     j = jn;
     cur = nxt;
     cur_w = nxt_w;
   }
+  if (HOLD) {
+    __syncthreads();
+    const int half_n = p.N >> 1;
+    auto flush = [&](int slot, int row0, int rows, int ct) {
+      const bf16_t *src = hold_base + slot * (BM * HOLD_ROW);
+      bf16_t *dst = reinterpret_cast<bf16_t *>(p.out) + (size_t)row0 * half_n + ct * (BN / 2);
+      for (int idx = threadIdx.x; idx < rows * 16; idx += GEMM_THREADS) {
+        const int row = idx >> 4, ch = (idx & 15) * 8;
+        if (ct * (BN / 2) + ch < half_n)
+          *reinterpret_cast<u32x4 *>(dst + (size_t)row * half_n + ch) =
+              *reinterpret_cast<const u32x4 *>(src + row * HOLD_ROW + ch);
+      }
+    };
+    flush(0, held_row0_a, held_rows_a, held_ct_a);
+    flush(1, held_row0_b, held_rows_b, held_ct_b);
+  }
 }
 
-template <int MBMAX>
+template <int MBMAX, bool HOLD = false>
 constexpr size_t gemm_smem_bytes() {
-  return (size_t)3 * MBMAX * 32 * LDS_ROW * sizeof(bf16_t);
+  return (size_t)3 * MBMAX * 32 * LDS_ROW * sizeof(bf16_t) + (HOLD ? (size_t)2 * MBMAX * 32 * HOLD_ROW * sizeof(bf16_t) : 0);
 }
 
 // The kernels use more dynamic LDS than a launch gets by default; the limit is raised for every
@@ -619,12 +672,12 @@ constexpr size_t gemm_smem_bytes() {
 template <int MBMAX, bool GATHER, int EPI, bool FP4>
 hipError_t gemm_set_attr() {
   return hipFuncSetAttribute(reinterpret_cast<const void *>(grouped_gemm_kernel<MBMAX, GATHER, EPI, FP4>),
-                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)gemm_smem_bytes<MBMAX>());
+                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)gemm_smem_bytes<MBMAX, gemm_holds_output(GATHER, EPI, FP4)>());
 }
 
 template <int MBMAX, bool GATHER, int EPI, bool FP4>
 int launch_gemm(const GemmParams &p, int max_tiles, hipStream_t s) {
-  const size_t smem = gemm_smem_bytes<MBMAX>();
+  const size_t smem = gemm_smem_bytes<MBMAX, gemm_holds_output(GATHER, EPI, FP4)>();
   auto kern = grouped_gemm_kernel<MBMAX, GATHER, EPI, FP4>;
   int total = max_tiles * p.n_col_tiles;
   int grid = ((total + 7) / 8) * 8;
