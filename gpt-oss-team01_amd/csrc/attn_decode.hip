@@ -1028,18 +1028,22 @@ static int attn_launch(const float *q, const void *kv_cache, const int *lens,
   int grid = (int)((items + 3) / 4) + (pl.wide ? 1 : 0);
   {
     TraceScope ts("attn_decode", s);
-    // one row per sequence: a resident grid that keeps its output rows in LDS until the end
+    // one row per sequence: a resident grid that keeps its output rows in LDS until the end (it
+    // writes them 16 bytes at a time; an output that is only 8-byte aligned gets the plain launch)
+    const bool hold_rows = !pair && aligned(out, 16);
     int resident = 0;
-    if (!pair) {
+    if (hold_rows) {
       const int rc = head_dim == 64 ? attn_resident_wgs<64>(&resident) : attn_resident_wgs<32>(&resident);
       if (rc != GPTOSS_OK) return rc;
     }
     if (head_dim == 64) {
       if (pair) attn_decode_kernel<64, true><<<grid, 256, 0, s>>>(p);
-      else attn_decode_resident_kernel<64><<<std::min(grid, resident), 256, 0, s>>>(p, grid);
+      else if (hold_rows) attn_decode_resident_kernel<64><<<std::min(grid, resident), 256, 0, s>>>(p, grid);
+      else attn_decode_kernel<64, false><<<grid, 256, 0, s>>>(p);
     } else {
       if (pair) attn_decode_kernel<32, true><<<grid, 256, 0, s>>>(p);
-      else attn_decode_resident_kernel<32><<<std::min(grid, resident), 256, 0, s>>>(p, grid);
+      else if (hold_rows) attn_decode_resident_kernel<32><<<std::min(grid, resident), 256, 0, s>>>(p, grid);
+      else attn_decode_kernel<32, false><<<grid, 256, 0, s>>>(p);
     }
   }
   GPTOSS_LAUNCH_CHECK("attn_decode_kernel");

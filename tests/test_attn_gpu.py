@@ -127,6 +127,31 @@ def test_attn_without_lengths_means_every_row_has_max_len(ops):
             assert torch.equal(a, b), (B, window)
 
 
+def test_attn_output_rows_kept_back_equal_rows_stored_at_once(ops):
+    """One query row per sequence and contexts of one chunk run on a resident grid that keeps its
+    output rows in LDS and writes them 16 bytes at a time after its last row; an output buffer that
+    is only 8-byte aligned gets the plain launch, which stores every row as it is finished.  Same bits
+    for a few rows (less than one round of the grid), for 1200 and for 8000 workgroup indices (several
+    rounds; the last case fills a workgroup's 16 slots and makes it write them in between), with
+    ragged lengths, empty rows and both head sizes."""
+    for B, n_q, n_kv, D, S in ((3, 8, 2, 32, 128), (600, 16, 8, 64, 192), (4000, 8, 8, 32, 128)):
+        q, K, V, sinks = _mk(B, S, n_q, n_kv, D, seed=33)
+        cache = ops.KVCache(B, n_kv, D, S)
+        cache.write(K.cuda(), V.cuda(), 0)
+        attn = ops.AttnDecode(B, n_q, n_kv, D, S)
+        g = torch.Generator().manual_seed(7)
+        lens = torch.randint(0, S + 1, (B,), generator=g, dtype=torch.int32)
+        lens[0] = S
+        lens = lens.cuda()
+        flat = torch.zeros(B * n_q * D + 8, dtype=torch.bfloat16, device="cuda")
+        for window in (0, 64):
+            a = attn.forward(q.cuda(), cache, lens, sinks.cuda(), window=window)
+            off = flat[4:4 + B * n_q * D].view(B, n_q, D)   # 8 bytes past a 16-byte boundary
+            assert off.data_ptr() % 16 == 8
+            attn.forward(q.cuda(), cache, lens, sinks.cuda(), window=window, out=off)
+            assert torch.equal(a, off), (B, D, window)
+
+
 def test_attn_bad_arguments(ops):
     import ctypes as C
     from conftest import load_pkg
